@@ -1,0 +1,309 @@
+// extern "C" kernel-level boundary (cx_*): argument checks, element-type dispatch, handle
+// life cycle.  Declarations and the reference interfaces they replace: include/comprex_gfx950.h.
+#include "cx_common.hpp"
+
+#include <cmath>
+
+namespace cx {
+
+std::string& last_error() {
+    static thread_local std::string msg;
+    return msg;
+}
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    last_error() = buf;
+    return code;
+}
+
+namespace {
+
+const char* status_text(int code) {
+    switch (code) {
+        case CX_ERR_MSG_TOO_LARGE: return "Decompression vector size is bigger than output buffer!";
+        case CX_ERR_CAPACITY: return "compressed message does not fit the buffer it was given";
+        case CX_ERR_INDEX: return "a message index lies outside the output vector";
+        case CX_ERR_INTERNAL: return "a bounded device-side wait expired";
+        default: return "device-side error";
+    }
+}
+
+// Reads and clears the device status word; waits for the stream.
+int collect_status(cx_handle h) {
+    CX_HIP(hipMemcpyAsync(h->h_pinned, h->d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, h->stream));
+    CX_HIP(hipStreamSynchronize(h->stream));
+    const int code = h->h_pinned[0];
+    if (code != 0) {
+        CX_HIP(hipMemsetAsync(h->d_status, 0, sizeof(DeviceStatus), h->stream));
+        CX_HIP(hipStreamSynchronize(h->stream));
+        return fail(code, "%s", status_text(code));
+    }
+    return CX_OK;
+}
+
+bool aligned4(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 3u) == 0; }
+
+}  // namespace
+}  // namespace cx
+
+using namespace cx;
+
+namespace {
+
+template <typename T>
+int finish_threshold(cx_handle h, T* d_thr_out, void* h_thr_out) {
+    if (!h_thr_out) return CX_OK;
+    const T* src = d_thr_out ? d_thr_out : static_cast<const T*>(h->d_thr);
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, src, sizeof(T), hipMemcpyDeviceToHost, h->stream));
+    int rc = collect_status(h);
+    memcpy(h_thr_out, h->h_pinned + 8, sizeof(T));
+    return rc;
+}
+
+template <typename T>
+int topk_threshold_impl(cx_handle h, const void* vec, const void* add_vec, int n, int add_n, float topK,
+                        int default_subsamples, float subsample_factor, void* d_thr_out, void* h_thr_out) {
+    if (add_vec && n != add_n) return fail(CX_ERR_SIZE_MISMATCH, "vector sizes must be the same!");
+    int subsamples = cx_topk_subsamples(topK, default_subsamples, subsample_factor);
+    if (subsamples < 0) subsamples = 0x7fffffff;  // undefined in the reference: use the whole vector
+    int rc;
+    if (n < subsamples) {
+        rc = launch_topk_threshold<T>(h, static_cast<const T*>(vec), static_cast<const T*>(add_vec), n, nullptr, n,
+                                      kSampleFull, 1.0f, topK, static_cast<T*>(d_thr_out));
+    } else {
+        const float stepsize = (float)n / (float)subsamples;
+        rc = launch_topk_threshold<T>(h, static_cast<const T*>(vec), static_cast<const T*>(add_vec), n, nullptr,
+                                      subsamples, kSampleStrided, stepsize, topK, static_cast<T*>(d_thr_out));
+    }
+    if (rc != CX_OK) return rc;
+    return finish_threshold<T>(h, static_cast<T*>(d_thr_out), h_thr_out);
+}
+
+template <typename T>
+int topk_threshold_indexed_impl(cx_handle h, const void* vec, const void* add_vec, int n, const int* d_idx, int m,
+                                float topK, void* d_thr_out, void* h_thr_out) {
+    int rc = launch_topk_threshold<T>(h, static_cast<const T*>(vec), static_cast<const T*>(add_vec), n, d_idx, m,
+                                      kSampleIndexed, 1.0f, topK, static_cast<T*>(d_thr_out));
+    if (rc != CX_OK) return rc;
+    return finish_threshold<T>(h, static_cast<T*>(d_thr_out), h_thr_out);
+}
+
+template <typename T>
+int compress_impl(cx_handle h, void* out_msg, long long out_capacity, const void* data, void* update, int n,
+                  const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
+    int rc = launch_compact<T>(h, out_msg, out_capacity, static_cast<const T*>(data), static_cast<T*>(update), n,
+                               static_cast<const T*>(thr_host), static_cast<const T*>(d_thr), d_size_prefix);
+    if (rc != CX_OK || !h_bytes) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, out_msg, 8, hipMemcpyDeviceToHost, h->stream));
+    rc = collect_status(h);
+    const int k = h->h_pinned[9];
+    *h_bytes = 8 + k * 4 * Elem<T>::pair_words;
+    return rc;
+}
+
+template <typename T>
+int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_bytes) {
+    int rc = launch_decompress<T>(h, static_cast<T*>(out), out_n, msg);
+    if (rc != CX_OK || !h_bytes) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
+    rc = collect_status(h);
+    *h_bytes = 8 + h->h_pinned[9] * 4 * Elem<T>::pair_words;
+    return rc;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* cx_last_error(void) { return last_error().c_str(); }
+
+int cx_abi_version(void) { return 1; }
+
+int cx_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
+int cx_pointer_on_device(const void* p) {
+    if (!p) return 0;
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();  // pageable host memory is reported as an error
+        return 0;
+    }
+    return (attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged ||
+            attr.type == hipMemoryTypeHost)
+               ? 1
+               : 0;
+}
+
+int cx_create(cx_handle* out, void* hip_stream) {
+    if (!out) return fail(CX_ERR_INVALID, "cx_create: null output");
+    *out = nullptr;
+    if (cx_device_count() < 1) return fail(CX_ERR_HIP, "cx_create: no HIP device available");
+    cx_handle h = new cx_handle_s();
+    h->stream = static_cast<hipStream_t>(hip_stream);
+    hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->tile_counter), 256);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->sel), sizeof(SelectState));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->d_status), 256);
+    if (e == hipSuccess) e = hipMalloc(&h->d_thr, 256);
+    if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&h->h_pinned), 64, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipMemset(h->tile_counter, 0, 256);
+    if (e == hipSuccess) e = hipMemset(h->sel, 0, sizeof(SelectState));
+    if (e == hipSuccess) e = hipMemset(h->d_status, 0, 256);
+    if (e == hipSuccess) e = hipMemset(h->d_thr, 0, 256);
+    if (e != hipSuccess) {
+        cx_destroy(h);
+        return fail(CX_ERR_HIP, "cx_create: %s", hipGetErrorString(e));
+    }
+    *out = h;
+    return CX_OK;
+}
+
+int cx_destroy(cx_handle h) {
+    if (!h) return CX_OK;
+    (void)hipStreamSynchronize(h->stream);
+    if (h->tile_desc) (void)hipFree(h->tile_desc);
+    if (h->tile_counter) (void)hipFree(h->tile_counter);
+    if (h->sel) (void)hipFree(h->sel);
+    if (h->d_status) (void)hipFree(h->d_status);
+    if (h->d_thr) (void)hipFree(h->d_thr);
+    if (h->h_pinned) (void)hipHostFree(h->h_pinned);
+    delete h;
+    return CX_OK;
+}
+
+int cx_set_stream(cx_handle h, void* hip_stream) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (h->stream != static_cast<hipStream_t>(hip_stream)) {
+        CX_HIP(hipStreamSynchronize(h->stream));  // scratch is shared between launches of one handle
+        h->stream = static_cast<hipStream_t>(hip_stream);
+    }
+    return CX_OK;
+}
+
+int cx_synchronize(cx_handle h) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    return collect_status(h);
+}
+
+int cx_set_option(cx_handle h, const char* key, int value) {
+    if (!h || !key) return fail(CX_ERR_INVALID, "null handle or key");
+    if (!strcmp(key, "compact_items")) {
+        if (value != 2 && value != 4 && value != 8) return fail(CX_ERR_INVALID, "compact_items must be 2, 4 or 8");
+        h->compact_items = value;
+    } else if (!strcmp(key, "compact_tile_ids")) {
+        if (value != 0 && value != 1) return fail(CX_ERR_INVALID, "compact_tile_ids must be 0 or 1");
+        h->compact_tile_ids = value;
+    } else if (!strcmp(key, "reduce_variant")) {
+        h->reduce_variant = value;
+    } else {
+        return fail(CX_ERR_INVALID, "unknown option '%s'", key);
+    }
+    return CX_OK;
+}
+
+void* cx_threshold_slot(cx_handle h) { return h ? h->d_thr : nullptr; }
+
+// ---- host arithmetic of ThresholdTopK (must reproduce the reference's fp32 steps) ----
+
+int cx_topk_subsamples(float topK, int default_subsamples, float subsample_factor) {
+    // `cond ? float : int` has type float: default_subsamples is rounded to fp32 first
+    const float req = subsample_factor / topK;
+    const float chosen = (req > (float)default_subsamples) ? req : (float)default_subsamples;
+    if (!(chosen < 2147483648.0f) || !(chosen > -2147483904.0f)) return -1;
+    return (int)chosen;
+}
+
+int cx_topk_pos(size_t m, float topK) {
+    const float prod = (float)m * topK;
+    const float up = std::ceil(prod);
+    const float minus = up - 1.0f;
+    return (int)minus;
+}
+
+#define CX_DISPATCH(dt, CALL)                                          \
+    switch (dt) {                                                      \
+        case CX_F32: { using T = float; return CALL; }                 \
+        case CX_F64: { using T = double; return CALL; }                \
+        case CX_I32: { using T = int; return CALL; }                   \
+        default: return fail(CX_ERR_INVALID, "unknown element type %d", (int)dt); \
+    }
+
+int cx_topk_threshold(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec, int n, int add_n, float topK,
+                      int default_subsamples, float subsample_factor, void* d_thr_out, void* h_thr_out) {
+    if (!h || n < 0 || (!vec && n > 0)) return fail(CX_ERR_INVALID, "topk_threshold: bad arguments");
+    if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
+    CX_DISPATCH(dt, topk_threshold_impl<T>(h, vec, add_vec, n, add_n, topK, default_subsamples, subsample_factor,
+                                           d_thr_out, h_thr_out));
+}
+
+int cx_topk_threshold_indexed(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec, int n, const int* d_idx,
+                              int m, float topK, void* d_thr_out, void* h_thr_out) {
+    if (!h || n < 0 || m < 0 || (!vec && n > 0) || (!d_idx && m > 0))
+        return fail(CX_ERR_INVALID, "topk_threshold_indexed: bad arguments");
+    if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
+    CX_DISPATCH(dt, topk_threshold_indexed_impl<T>(h, vec, add_vec, n, d_idx, m, topK, d_thr_out, h_thr_out));
+}
+
+int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
+                   int n, const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, compress_impl<T>(h, out_msg, out_capacity, data, update, n, thr_host, d_thr, d_size_prefix, h_bytes));
+}
+
+int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (!aligned4(msg)) return fail(CX_ERR_INVALID, "message must be 4-byte aligned");
+    CX_DISPATCH(dt, decompress_impl<T>(h, out, out_n, msg, h_bytes));
+}
+
+int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int check) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (!msg || !aligned4(msg)) return fail(CX_ERR_INVALID, "message must be a 4-byte aligned device pointer");
+    if (check) {
+        CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->h_pinned[8] > out_n)
+            return fail(CX_ERR_MSG_TOO_LARGE, "Decompression vector size is bigger than output buffer!");
+    }
+    CX_DISPATCH(dt, launch_add<T>(h, static_cast<T*>(out), out_n, msg, 0));
+}
+
+int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* const* msgs, int n_msgs, int accumulate,
+                 int mode) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    for (int r = 0; r < n_msgs; ++r)
+        if (!msgs || !msgs[r] || !aligned4(msgs[r]))
+            return fail(CX_ERR_INVALID, "message %d must be a 4-byte aligned device pointer", r);
+    CX_DISPATCH(dt, launch_reduce<T>(h, static_cast<T*>(out), out_n, msgs, n_msgs, accumulate, mode));
+}
+
+int cx_zero(cx_handle h, cx_dtype dt, void* v, int n) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, launch_zero<T>(h, static_cast<T*>(v), n));
+}
+
+int cx_add_vec(cx_handle h, cx_dtype dt, void* data, const void* rests, int n) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, launch_add_vec<T>(h, static_cast<T*>(data), static_cast<const T*>(rests), n));
+}
+
+int cx_threshold_apply(cx_handle h, cx_dtype dt, void* high, void* low, const void* in, int n, const void* thr_host,
+                       const void* d_thr) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, launch_threshold_apply<T>(h, static_cast<T*>(high), static_cast<T*>(low), static_cast<const T*>(in),
+                                              n, static_cast<const T*>(thr_host), static_cast<const T*>(d_thr)));
+}
+
+}  // extern "C"

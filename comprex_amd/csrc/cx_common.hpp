@@ -1,0 +1,113 @@
+// Shared host-side declarations of the gfx950 library: handle layout, error plumbing,
+// element-type traits.  Device code lives in the k_*.hip files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/comprex_gfx950.h"
+
+namespace cx {
+
+// ---- error plumbing --------------------------------------------------------
+std::string& last_error();
+int fail(int code, const char* fmt, ...);
+
+#define CX_HIP(call)                                                                         \
+    do {                                                                                     \
+        hipError_t e__ = (call);                                                             \
+        if (e__ != hipSuccess)                                                               \
+            return ::cx::fail(CX_ERR_HIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(e__), \
+                              __FILE__, __LINE__);                                           \
+    } while (0)
+
+// ---- per-element-type traits -----------------------------------------------
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    using key_t = uint32_t;
+    static constexpr int key_bits = 31;  // sign stripped
+    static constexpr int pair_words = 2;
+};
+template <> struct Elem<int> {
+    using key_t = uint32_t;
+    static constexpr int key_bits = 32;  // |INT_MIN| needs bit 31
+    static constexpr int pair_words = 2;
+};
+template <> struct Elem<double> {
+    using key_t = uint64_t;
+    static constexpr int key_bits = 63;
+    static constexpr int pair_words = 3;
+};
+
+// ---- device-side scratch layouts -------------------------------------------
+constexpr int kRadixBits = 11;
+constexpr int kRadixBins = 1 << kRadixBits;
+
+// State of one radix-select run; lives in device memory.
+struct SelectState {
+    unsigned long long prefix;     // key bits fixed so far
+    unsigned long long mask;       // which bits of `prefix` are fixed
+    unsigned long long rank;       // descending rank still to find among matching keys
+    unsigned int hist[kRadixBins]; // digit histogram of the current pass
+};
+
+// Device status word: first error wins.
+struct DeviceStatus {
+    int code;
+    int detail;
+};
+
+}  // namespace cx
+
+// The handle: stream + scratch of one compressor clone.
+struct cx_handle_s {
+    int device = 0;
+    hipStream_t stream = nullptr;
+
+    // ordered-compaction scratch: one 64-bit descriptor per tile + the dynamic tile counter
+    unsigned long long* tile_desc = nullptr;
+    size_t tile_desc_cap = 0;          // descriptors allocated
+    unsigned int* tile_counter = nullptr;
+    unsigned int counter_base = 0;     // value of *tile_counter before the next launch
+    unsigned int epoch = 0;            // launch number stamped into descriptors
+
+    cx::SelectState* sel = nullptr;
+    cx::DeviceStatus* d_status = nullptr;
+    void* d_thr = nullptr;             // 8-byte threshold slot
+    int* h_pinned = nullptr;           // 64-byte pinned read-back area
+
+    // options
+    int compact_items = 4;             // vector loads per thread and tile
+    int compact_tile_ids = 0;          // 0 = dynamic tile counter, 1 = blockIdx order
+    int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
+};
+
+namespace cx {
+
+// ---- launchers implemented in the k_*.hip files -----------------------------
+template <typename T>
+int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
+                   const T* thr_host, const T* d_thr, int* d_size_prefix);
+
+template <typename T>
+int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m,
+                          int sample_mode, float stepsize, float topK, T* d_thr_out);
+
+template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg);
+template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);
+template <typename T>
+int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode);
+template <typename T> int launch_zero(cx_handle h, T* v, int n);
+template <typename T> int launch_add_vec(cx_handle h, T* data, const T* rests, int n);
+template <typename T>
+int launch_threshold_apply(cx_handle h, T* high, T* low, const T* in, int n, const T* thr_host, const T* d_thr);
+
+// sample_mode of launch_topk_threshold
+enum { kSampleFull = 0, kSampleStrided = 1, kSampleIndexed = 2 };
+
+}  // namespace cx

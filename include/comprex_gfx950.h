@@ -1,0 +1,195 @@
+/*
+ * comprex_gfx950.h -- C ABI of the MI355X (gfx950) implementation of ComprEx's
+ * gradient-compression hot path.
+ *
+ * Two groups of entry points live in libcomprex_gfx950.so:
+ *
+ *  1. cx_*  : the kernel-level boundary.  Plain pointers and sizes, no C++ or torch
+ *             types.  Vectors and messages are DEVICE pointers (anything the GPU can
+ *             dereference); scalars are passed by value or through small host
+ *             pointers.  Each function cites the reference interface it replaces
+ *             (paths relative to the reference tree).  Calls are enqueued on the
+ *             handle's HIP stream and return without waiting unless a host output
+ *             pointer is given.
+ *
+ *  2. The reference's own float-only symbol set (src/comprEx_C.cpp:17-87,
+ *     src/GPI_C.cpp:41-73, src/allreduce_C.cpp:26-122), so that the reference's
+ *     ctypes wrappers bind unchanged; declared at the end of this file.
+ *
+ * Element types: the reference's templates are instantiated for float in its C ABI
+ * (src/comprEx_C.cpp:12) and for int in its tests (test/compressor.cpp:8); double is
+ * allowed by the templates.  All three are supported here (cx_dtype).
+ *
+ * Message layout (src/compressor.hxx:559-565,606), unchanged:
+ *     int32 n (uncompressed length) | int32 k (pairs) | k x { int32 index, T value }
+ * pairs packed without padding, indices strictly ascending.
+ */
+#ifndef COMPREX_GFX950_H
+#define COMPREX_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cx_handle_s* cx_handle;
+
+typedef enum { CX_F32 = 0, CX_F64 = 1, CX_I32 = 2 } cx_dtype;
+
+typedef enum {
+    CX_OK = 0,
+    CX_ERR_INVALID = 1,        /* bad argument (null pointer, negative size, unknown dtype) */
+    CX_ERR_SIZE_MISMATCH = 2,  /* vector sizes differ (reference: throws, compressor.hxx:45-49, threshold.hxx:161-163) */
+    CX_ERR_MSG_TOO_LARGE = 3,  /* message's vector length exceeds the output (compressor.hxx:620-624,645-647) */
+    CX_ERR_CAPACITY = 4,       /* message would not fit the caller's buffer (the reference overruns silently) */
+    CX_ERR_INDEX = 5,          /* a pair's index lies outside the output vector (the reference overruns silently) */
+    CX_ERR_HIP = 6,            /* a HIP runtime call failed */
+    CX_ERR_INTERNAL = 7,       /* a bounded device-side wait expired */
+    CX_ERR_TOPK = 8            /* topK outside [0,1] (threshold.hxx:131-133) */
+} cx_status;
+
+/* Text of the last error raised on the calling thread. */
+const char* cx_last_error(void);
+/* ABI version of this header. */
+int cx_abi_version(void);
+/* Number of HIP devices visible (0 when there is no GPU); never throws. */
+int cx_device_count(void);
+/* 1 when `p` is device (or managed/host-registered) memory, 0 for pageable host memory. */
+int cx_pointer_on_device(const void* p);
+
+/* A handle owns one HIP stream reference and the scratch memory of one compressor
+ * clone (tile descriptors, histograms, a device-side threshold slot, a status word).
+ * It replaces the per-object state of Compressor<T>/ThresholdFunction<T> clones
+ * (src/comprEx.tpp:94-112).  Not thread safe, like the reference's objects. */
+int cx_create(cx_handle* out, void* hip_stream /* hipStream_t, NULL = default stream */);
+int cx_destroy(cx_handle h);
+int cx_set_stream(cx_handle h, void* hip_stream);
+/* Waits for the handle's stream and returns the first device-side error seen since the
+ * last call (CX_OK if none), clearing it. */
+int cx_synchronize(cx_handle h);
+/* Tuning switches (compaction tile and ordering variant, reduce variant); see the .md
+ * design notes of the source tree.  Unknown keys return CX_ERR_INVALID. */
+int cx_set_option(cx_handle h, const char* key, int value);
+
+/* ---- thresholds ----------------------------------------------------------- */
+
+/* ThresholdTopK<T>::calc_subsamples (src/threshold.hxx:182-186).  -1 where the
+ * reference's float->int conversion is undefined. */
+int cx_topk_subsamples(float topK, int default_subsamples, float subsample_factor);
+/* topk_pos of ThresholdTopK<T>::calc_threshold (src/threshold.hxx:190). */
+int cx_topk_pos(size_t m, float topK);
+
+/* ThresholdTopK<T>::prepare_with(vec, n, add_vec, n) / prepare(vec, n) when add_vec is
+ * NULL (src/threshold.hxx:152-167): strided sub-sample (or the whole vector when
+ * n < subsamples) of vec[p] + add_vec[p], then the (topk_pos+1)-th largest magnitude
+ * (or max+1 when topk_pos <= 0).  The threshold is written to `d_thr_out` (device, T;
+ * NULL = the handle's own slot, see cx_threshold_slot) and, when `h_thr_out` is not
+ * NULL, also copied to the host (this waits for the stream). */
+int cx_topk_threshold(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec, int n, int add_n,
+                      float topK, int default_subsamples, float subsample_factor,
+                      void* d_thr_out, void* h_thr_out);
+/* Same order statistic over m host-chosen sample positions d_idx[0..m) (device int32):
+ * keys are vec[idx] (+ add_vec[idx]).  No counterpart in the reference, whose sampling
+ * is always strided (src/threshold.hxx:224-240); calc_threshold (:189-205) is unchanged. */
+int cx_topk_threshold_indexed(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec,
+                              int n, const int* d_idx, int m, float topK, void* d_thr_out, void* h_thr_out);
+/* Device address of the handle's threshold slot (8 bytes, holds a T). */
+void* cx_threshold_slot(cx_handle h);
+
+/* ---- IndexPairs codec ------------------------------------------------------ */
+
+/* CompressorIndexPairs<T>::compression_strategy (src/compressor.hxx:556-611) behind
+ * Compressor<T>::compress / compress_update / compress_add_update (:36-51):
+ *   data != NULL, update != NULL : update += data; emit |update| > thr; zero emitted
+ *   data == NULL                 : emit |update| > thr; zero emitted
+ *   update == NULL               : emit |data| > thr
+ * `out_msg` needs 4-byte alignment only.  The threshold comes from `thr_host`
+ * (pointer to a host T) or, when that is NULL, from `d_thr` (device T; NULL = the
+ * handle's slot).  `out_capacity` is the size in bytes of out_msg: pairs beyond it are
+ * not written and CX_ERR_CAPACITY is recorded.  `d_size_prefix` (device int32, may be
+ * NULL) receives the message's byte count (the send_sizeBytes prefix of
+ * src/comprEx.tpp:184-188).  When `h_bytes` is not NULL the call waits and stores the
+ * bytes written (8 + k*(4+sizeof(T))), as the reference returns them. */
+int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity,
+                   const void* data, void* update, int n,
+                   const void* thr_host, const void* d_thr,
+                   int* d_size_prefix, int* h_bytes);
+
+/* CompressorIndexPairs<T>::decompression_strategy (src/compressor.hxx:613-638): zero
+ * all out_n elements, then out[index] = value.  A message whose n exceeds out_n leaves
+ * `out` zeroed and records CX_ERR_MSG_TOO_LARGE.  h_bytes as above (bytes consumed). */
+int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes);
+
+/* CompressorIndexPairs<T>::add_strategy (src/compressor.hxx:640-658): out[index] += value
+ * in message order.  A message whose n exceeds out_n changes nothing and records
+ * CX_ERR_MSG_TOO_LARGE.  `check` != 0 reads the header first and returns that error
+ * synchronously, as the reference throws before touching `out`. */
+int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int check);
+
+/* The chief's reduce loop of Comprex_AllToOneAllreduce::apply (src/allreduce.tpp:183-189):
+ * out (+)= sum over messages in the order given.  `msgs` is a HOST array of n_msgs device
+ * pointers.  accumulate == 0 starts from zero (decompress of the first message followed by
+ * add of the rest), != 0 adds into `out`.  mode 0 = rank-ordered, bit-exact; mode 1 =
+ * floating-point atomics (order of additions unspecified). */
+int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* const* msgs, int n_msgs,
+                 int accumulate, int mode);
+
+/* ---- residual maintenance -------------------------------------------------- */
+
+/* ComprEx<T>::resetRests (src/comprEx.tpp:121-126): v[0..n) = 0. */
+int cx_zero(cx_handle h, cx_dtype dt, void* v, int n);
+/* ComprEx<T>::addRests (src/comprEx.tpp:159-169): data[i] += rests[i]. */
+int cx_add_vec(cx_handle h, cx_dtype dt, void* data, const void* rests, int n);
+/* ThresholdFunction<T>::apply with a given threshold (src/threshold.hxx:19-27):
+ * out = |in| >= thr ? in : 0, and apply_split (:30-50) when `low` is not NULL. */
+int cx_threshold_apply(cx_handle h, cx_dtype dt, void* high, void* low, const void* in, int n,
+                       const void* thr_host, const void* d_thr);
+
+/* ---- the reference's C ABI (float only) ------------------------------------- */
+/* src/GPI_C.cpp:41-73.  One process stands for `ranks` simulated ranks that exchange
+ * messages through device buffers; segment_size is accepted and ignored. */
+void* GaspiEnvironment_new(int segment_size);
+void GaspiEnvironment_del(void* self);
+int GaspiEnvironment_get_rank(void* self);
+int GaspiEnvironment_get_ranks(void* self);
+void GaspiEnvironment_barrier(void* self);
+void GaspiEnvironment_flush(void* self);
+void Gaspi_Printf(const char* msg);
+/* Not in the reference: selects which simulated rank the next calls act as, and how many
+ * there are (the reference gets both from gaspi_run). */
+void GaspiEnvironment_set_rank(void* self, int rank, int ranks);
+
+/* src/comprEx_C.cpp:17-87 */
+void* Comprex_new(void* gaspi_env, int size, float size_factor);
+void Comprex_del(void* self);
+void Comprex_setThreshold(void* self, const void* threshold);
+void Comprex_setCompressor(void* self, const void* compressor);
+void Comprex_resetRests(void* self);
+void Comprex_flushRests(void* self);
+void Comprex_getRests(void* self, float* vector, int size);
+void Comprex_writeRemote(void* self, const float* vector, int size);
+void Comprex_readRemote(void* self, float* vector, int size);
+void Comprex_readRemote_add(void* self, float* vector, int size);
+void Comprex_connectTo(void* self, int srcRank, int targRank, int tag);
+void Comprex_connectTx(void* self, int targRank, int tag);
+void Comprex_connectRx(void* self, int srcRank, int tag);
+void* ThresholdNone_new(void);
+void ThresholdNone_del(void* self);
+void* ThresholdConst_new(float thr);
+void ThresholdConst_del(void* self);
+float ThresholdConst_getThreshold(void* self);
+void* ThresholdTopK_new(float topK);
+void ThresholdTopK_del(void* self);
+float ThresholdTopK_getThreshold(void* self);
+void* CompressorIndexPairs_new(void);
+void CompressorIndexPairs_del(void* self);
+/* Error text of the last reference-ABI call that failed on this thread ("" if none).  The
+ * reference lets std::runtime_error escape through extern "C"; here it is caught. */
+const char* Comprex_lastError(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

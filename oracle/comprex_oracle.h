@@ -1,0 +1,120 @@
+/*
+ * comprex_oracle.h -- CPU restatement of ComprEx's compression hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is the checker the HIP kernels are compared
+ * against; nothing in the product library links, loads or calls it.  Only the
+ * test-suite, the smoke check and the CPU-baseline leg of the benchmark may use
+ * it.  Plain C, single threaded, written from the semantics of the reference
+ * sources (paths below are relative to the reference tree):
+ *
+ *   src/threshold.hxx:127-242   ThresholdTopK (sub-sampling, order statistic)
+ *   src/threshold.hxx:96-119    ThresholdConst, :72-88 ThresholdNone
+ *   src/threshold.hxx:19-50     ThresholdFunction::apply / apply_split
+ *   src/compressor.hxx:24-76    Compressor wrappers (size check)
+ *   src/compressor.hxx:538-661  CompressorIndexPairs (compress / decompress / add)
+ *   src/comprEx.tpp:121-246     residual maintenance, writeRemote*, flushRests, readRemote*
+ *
+ * Every function is pinned (tests/test_oracle_*.py) against: the compiled
+ * reference headers (oracle/_ref, when the reference tree is present), the
+ * known answers of the reference's own tests (test/threshold.cpp,
+ * test/compressor.cpp, test/comprex.cpp), brute-force sorting on small inputs
+ * and the committed fixtures under tests/golden/.
+ *
+ * Parity unpinned (undefined behaviour in the reference, so there is nothing to
+ * pin): inputs containing NaN in the threshold computation (the reference's
+ * nth_element comparator is not a strict weak order for NaN); topK == 0 and
+ * empty vectors in ThresholdTopK (the reference converts +inf to int / dereferences
+ * end()).  The oracle returns a defined value for these and says which below.
+ *
+ * Three element types are instantiated, as in the reference's templates:
+ *   f32 (float), f64 (double), i32 (int; the type the reference's tests use).
+ */
+#ifndef COMPREX_ORACLE_H
+#define COMPREX_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- type independent host arithmetic ---------------------------------- */
+
+/* threshold.hxx:182-186 calc_subsamples(): fp32 quotient, float/int ternary
+ * (common type float), truncation to int.  Returns -1 where the reference's
+ * conversion is undefined (topK == 0 gives +inf, or a value beyond INT_MAX). */
+int cxo_calc_subsamples(float topK, int default_subsamples, float subsample_factor);
+
+/* threshold.hxx:190 topk_pos = ceil(size * topK) - 1 with the product, the
+ * ceil and the "- 1" all evaluated in fp32 before the conversion to int. */
+int cxo_topk_pos(size_t m, float topK);
+
+/* threshold.hxx:214-219 / :233-238: position of sample i of `subsamples`
+ * strided samples over a vector of n elements: (int)(i * ((float)n/(float)subsamples)),
+ * the product evaluated in fp32. */
+int cxo_strided_pos(int i, int n, int subsamples);
+
+/* number of keys the threshold is computed on: n when n < subsamples (strict,
+ * threshold.hxx:210,226), else subsamples. */
+int cxo_sample_count(int n, int subsamples);
+
+#define CXO_DECLARE(SFX, T)                                                                   \
+    /* threshold.hxx:189-205 calc_threshold on a scratch copy (reordered in place).          \
+     * m == 0 is undefined in the reference; the oracle returns 1. */                        \
+    T cxo_calc_threshold_##SFX(T* vec_copy, size_t m, float topK);                            \
+    /* threshold.hxx:152-156 prepare(vec): prep_vec (:208-221) then calc_threshold. */        \
+    T cxo_topk_prepare_##SFX(const T* vec, int n, float topK, int default_subsamples,         \
+                             float subsample_factor);                                         \
+    /* threshold.hxx:160-167 prepare_with(vec, add_vec): prep_add_vec (:224-240) then         \
+     * calc_threshold.  Returns 0 and sets *err=1 when sizes differ (reference throws). */    \
+    T cxo_topk_prepare_with_##SFX(const T* vec, int n, const T* add_vec, int add_n,           \
+                                  float topK, int default_subsamples,                         \
+                                  float subsample_factor, int* err);                          \
+    /* Variant with host-supplied sample positions (not in the reference: the same            \
+     * calc_threshold applied to vec[idx[i]] (+ add_vec[idx[i]] when add_vec != NULL)). */    \
+    T cxo_topk_prepare_indexed_##SFX(const T* vec, const T* add_vec, const int* idx, int m,   \
+                                     float topK);                                             \
+    /* threshold.hxx:19-27 apply(): out = |in| >= thr ? in : 0  (note >=). */                 \
+    void cxo_threshold_apply_##SFX(T* out, const T* in, int n, T thr);                        \
+    /* threshold.hxx:30-50 apply_split(). */                                                  \
+    void cxo_threshold_apply_split_##SFX(T* high, T* low, const T* in, int n, T thr);         \
+    /* compressor.hxx:556-611 compression_strategy.  data and/or update may be NULL:          \
+     * both -> fused (update += data, select, emit, zero); update only; data only.            \
+     * Returns bytes written (8 + k*(4+sizeof(T))), or -1 when both are NULL                  \
+     * (the reference writes an empty message in that case; see .c). */                       \
+    int cxo_ip_compress_##SFX(void* out, const T* data, T* update, int n, T thr);             \
+    /* compressor.hxx:44-51 compress_add_update size check; -2 on mismatch (reference throws) */\
+    int cxo_ip_compress_add_update_##SFX(void* out, T* update, int update_n, const T* data,   \
+                                         int data_n, T thr);                                  \
+    /* compressor.hxx:613-638 decompression_strategy: zero all out_n, scatter.  Returns       \
+     * bytes consumed, or -1 when the message's vector size exceeds out_n (reference          \
+     * throws after the memset, so out is zeroed in that case too). */                        \
+    int cxo_ip_decompress_##SFX(T* out, int out_n, const void* in);                           \
+    /* compressor.hxx:640-658 add_strategy: out[idx] += val in message order.  Returns 0,     \
+     * or -1 when the message's vector size exceeds out_n (nothing modified). */              \
+    int cxo_ip_add_##SFX(T* out, int out_n, const void* in);                                  \
+    /* comprEx.tpp:159-169 addRests: data[i] += rests[i]. */                                  \
+    void cxo_add_rests_##SFX(T* data, const T* rests, int n);                                 \
+    /* comprEx.tpp:176-191 writeRemote: prepare_with + compress_add_update into               \
+     * buf (+4 when send_size_bytes, the int prefix then holds the message bytes).            \
+     * Returns message bytes (without the prefix). */                                         \
+    int cxo_write_remote_##SFX(void* buf, int send_size_bytes, T* rests, const T* vec, int n, \
+                               float topK, int default_subsamples, float subsample_factor,    \
+                               T* thr_out);                                                   \
+    /* comprEx.tpp:208-222 writeRemote_NoResidual: prepare(vec) + data-only compress. */      \
+    int cxo_write_remote_noresidual_##SFX(void* buf, int send_size_bytes, const T* vec, int n,\
+                                          float topK, int default_subsamples,                 \
+                                          float subsample_factor, T* thr_out);                \
+    /* comprEx.tpp:128-142 flushRests: data-only compress of rests at threshold 0, then       \
+     * zero the residual. */                                                                  \
+    int cxo_flush_rests_##SFX(void* buf, int send_size_bytes, T* rests, int n);
+
+CXO_DECLARE(f32, float)
+CXO_DECLARE(f64, double)
+CXO_DECLARE(i32, int)
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,219 @@
+"""ctypes doorway onto the CPU checker libraries.
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, ``__graft_entry__.smoke()`` and
+the ``cpu_baseline`` leg of ``bench.py``; the product package never imports it.
+
+``Oracle()``      -> liboracle.so, the plain-C restatement (``cxo_*`` symbols)
+``Oracle(ref=True)`` -> _ref/libref.so, the reference's own headers behind an
+                     extern "C" shim (``cxr_*`` symbols); present only where it was
+                     built from the reference tree.
+
+Both expose the same methods; arrays are 1-D contiguous numpy arrays of dtype
+float32 / float64 / int32, messages are ``np.uint8`` buffers.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SFX = {np.dtype(np.float32): "f32", np.dtype(np.float64): "f64", np.dtype(np.int32): "i32"}
+_CT = {"f32": C.c_float, "f64": C.c_double, "i32": C.c_int}
+
+
+def build():
+    """Compile liboracle.so (and _ref/libref.so when the reference tree is here)."""
+    subprocess.run(["make", "-C", _HERE, "all"], check=True, capture_output=True)
+
+
+def ref_available():
+    return os.path.exists(os.path.join(_HERE, "_ref", "libref.so"))
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class Oracle:
+    def __init__(self, ref=False):
+        self.ref = ref
+        path = os.path.join(_HERE, "_ref", "libref.so") if ref else os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(path):
+            if ref:
+                raise FileNotFoundError(path)
+            build()
+        self.lib = C.CDLL(path)
+        self.p = "cxr_" if ref else "cxo_"
+        self.kind = "reference" if ref else "port"
+
+    # ---- helpers -------------------------------------------------------
+    def _f(self, name, restype, *argtypes):
+        fn = getattr(self.lib, self.p + name)
+        fn.restype = restype
+        fn.argtypes = list(argtypes)
+        return fn
+
+    @staticmethod
+    def _sfx(a):
+        a = np.asarray(a)
+        assert a.flags["C_CONTIGUOUS"], "oracle arrays must be contiguous"
+        return _SFX[a.dtype]
+
+    # ---- host arithmetic ----------------------------------------------
+    def calc_subsamples(self, topK, default_subsamples=1000, subsample_factor=10.0):
+        return self._f("calc_subsamples", C.c_int, C.c_float, C.c_int, C.c_float)(
+            topK, default_subsamples, subsample_factor)
+
+    def topk_pos(self, m, topK):
+        assert not self.ref
+        return self._f("topk_pos", C.c_int, C.c_size_t, C.c_float)(m, topK)
+
+    def strided_pos(self, i, n, subsamples):
+        assert not self.ref
+        return self._f("strided_pos", C.c_int, C.c_int, C.c_int, C.c_int)(i, n, subsamples)
+
+    # ---- thresholds ---------------------------------------------------
+    def calc_threshold(self, vec, topK):
+        s = self._sfx(vec)
+        scratch = vec.copy()
+        return self._f("calc_threshold_" + s, _CT[s], C.c_void_p, C.c_size_t, C.c_float)(
+            _ptr(scratch), scratch.size, topK)
+
+    def topk_prepare(self, vec, topK, default_subsamples=1000, subsample_factor=10.0):
+        s = self._sfx(vec)
+        return self._f("topk_prepare_" + s, _CT[s], C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float)(
+            _ptr(vec), vec.size, topK, default_subsamples, subsample_factor)
+
+    def topk_prepare_with(self, vec, add_vec, topK, default_subsamples=1000, subsample_factor=10.0):
+        s = self._sfx(vec)
+        err = C.c_int(0)
+        thr = self._f("topk_prepare_with_" + s, _CT[s], C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                      C.c_float, C.c_int, C.c_float, C.POINTER(C.c_int))(
+            _ptr(vec), vec.size, _ptr(add_vec), add_vec.size, topK, default_subsamples,
+            subsample_factor, C.byref(err))
+        if err.value:
+            raise RuntimeError("vector sizes must be the same!")
+        return thr
+
+    def topk_prepare_indexed(self, vec, add_vec, idx, topK):
+        assert not self.ref
+        s = self._sfx(vec)
+        idx = np.ascontiguousarray(idx, dtype=np.int32)
+        return self._f("topk_prepare_indexed_" + s, _CT[s], C.c_void_p, C.c_void_p, C.c_void_p,
+                       C.c_int, C.c_float)(_ptr(vec), _ptr(add_vec), _ptr(idx), idx.size, topK)
+
+    def threshold_apply(self, vec, thr):
+        s = self._sfx(vec)
+        out = np.empty_like(vec)
+        self._f("threshold_apply_" + s, None, C.c_void_p, C.c_void_p, C.c_int, _CT[s])(
+            _ptr(out), _ptr(vec), vec.size, thr)
+        return out
+
+    def threshold_apply_split(self, vec, thr):
+        s = self._sfx(vec)
+        hi, lo = np.empty_like(vec), np.empty_like(vec)
+        self._f("threshold_apply_split_" + s, None, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _CT[s])(
+            _ptr(hi), _ptr(lo), _ptr(vec), vec.size, thr)
+        return hi, lo
+
+    def topk_apply(self, vec, topK):
+        """ThresholdTopK(topK).apply (reference shim only): (masked copy, threshold)."""
+        assert self.ref
+        s = self._sfx(vec)
+        out = np.empty_like(vec)
+        thr = self._f("topk_apply_" + s, _CT[s], C.c_void_p, C.c_void_p, C.c_int, C.c_float)(
+            _ptr(out), _ptr(vec), vec.size, topK)
+        return out, thr
+
+    # ---- IndexPairs codec --------------------------------------------
+    @staticmethod
+    def message_capacity(n, dtype):
+        return 8 + n * (4 + np.dtype(dtype).itemsize)
+
+    def ip_compress(self, data, update, thr, out=None):
+        """data and/or update (update is modified in place).  Returns the message bytes."""
+        ref_arr = data if data is not None else update
+        s = self._sfx(ref_arr)
+        n = ref_arr.size
+        if out is None:
+            out = np.zeros(self.message_capacity(n, ref_arr.dtype), dtype=np.uint8)
+        nbytes = self._f("ip_compress_" + s, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _CT[s])(
+            _ptr(out), _ptr(data), _ptr(update), n, thr)
+        return out[:nbytes]
+
+    def ip_compress_add_update(self, update, data, thr):
+        s = self._sfx(update)
+        out = np.zeros(self.message_capacity(max(update.size, data.size), update.dtype), dtype=np.uint8)
+        nbytes = self._f("ip_compress_add_update_" + s, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
+                         C.c_void_p, C.c_int, _CT[s])(
+            _ptr(out), _ptr(update), update.size, _ptr(data), data.size, thr)
+        if nbytes == -2:
+            raise RuntimeError("Compressor: Update vector size (%d) is not equal data vector size (%d)!"
+                               % (update.size, data.size))
+        return out[:nbytes]
+
+    def ip_decompress(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("ip_decompress_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(
+            _ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+        return r
+
+    def ip_add(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("ip_add_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(_ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+
+    # ---- channel level (restatement only) ----------------------------
+    def add_rests(self, data, rests):
+        assert not self.ref
+        s = self._sfx(data)
+        self._f("add_rests_" + s, None, C.c_void_p, C.c_void_p, C.c_int)(_ptr(data), _ptr(rests), data.size)
+
+    def write_remote(self, rests, vec, topK, default_subsamples=1000, subsample_factor=10.0,
+                     send_size_bytes=False):
+        """Returns (buffer bytes incl. optional prefix, threshold)."""
+        assert not self.ref
+        s = self._sfx(vec)
+        buf = np.zeros(4 + self.message_capacity(vec.size, vec.dtype), dtype=np.uint8)
+        thr = _CT[s]()
+        nbytes = self._f("write_remote_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                         C.c_int, C.c_float, C.c_int, C.c_float, C.c_void_p)(
+            _ptr(buf), int(send_size_bytes), _ptr(rests), _ptr(vec), vec.size, topK,
+            default_subsamples, subsample_factor, C.byref(thr))
+        return buf[:nbytes + (4 if send_size_bytes else 0)], thr.value
+
+    def write_remote_noresidual(self, vec, topK, default_subsamples=1000, subsample_factor=10.0,
+                                send_size_bytes=False):
+        assert not self.ref
+        s = self._sfx(vec)
+        buf = np.zeros(4 + self.message_capacity(vec.size, vec.dtype), dtype=np.uint8)
+        thr = _CT[s]()
+        nbytes = self._f("write_remote_noresidual_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p,
+                         C.c_int, C.c_float, C.c_int, C.c_float, C.c_void_p)(
+            _ptr(buf), int(send_size_bytes), _ptr(vec), vec.size, topK, default_subsamples,
+            subsample_factor, C.byref(thr))
+        return buf[:nbytes + (4 if send_size_bytes else 0)], thr.value
+
+    def flush_rests(self, rests, send_size_bytes=False):
+        assert not self.ref
+        s = self._sfx(rests)
+        buf = np.zeros(4 + self.message_capacity(rests.size, rests.dtype), dtype=np.uint8)
+        nbytes = self._f("flush_rests_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int)(
+            _ptr(buf), int(send_size_bytes), _ptr(rests), rests.size)
+        return buf[:nbytes + (4 if send_size_bytes else 0)]
+
+
+def parse_message(msg, dtype):
+    """Split an IndexPairs message into (n, k, indices int32[k], values dtype[k])."""
+    msg = np.ascontiguousarray(msg, dtype=np.uint8)
+    n, k = np.frombuffer(msg[:8].tobytes(), dtype=np.int32)
+    dt = np.dtype(dtype)
+    rec = np.dtype([("i", np.int32), ("v", dt)], align=False)
+    body = np.frombuffer(msg[8:8 + int(k) * rec.itemsize].tobytes(), dtype=rec)
+    return int(n), int(k), body["i"].copy(), body["v"].copy()

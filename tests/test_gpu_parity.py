@@ -1,0 +1,362 @@
+"""Parity of the HIP path with the CPU checker, through the C ABI, on one MI355X.
+
+Bit-exact bar: thresholds, index sets, pair order, residuals, dense outputs of the
+rank-ordered reduce.  Tolerance bar (stated where used): the atomic reduce variant.
+"""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.pyoracle import parse_message
+
+pytestmark = pytest.mark.gpu
+
+NP2T = {np.float32: torch.float32, np.float64: torch.float64, np.int32: torch.int32}
+DTYPES = [np.float32, np.float64, np.int32]
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from comprex_amd.device import Handle
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    h = Handle()
+    yield h
+    h.synchronize()
+    h.close()
+
+
+def _rand(rng, n, dtype, scale=1.0):
+    if dtype == np.int32:
+        return rng.integers(-1000, 1001, n).astype(np.int32)
+    return (rng.standard_normal(n) * scale).astype(dtype)
+
+
+def _gpu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _msgbuf(n, dtype, extra=0):
+    from comprex_amd.device import message_capacity
+    return torch.zeros(message_capacity(n, NP2T[dtype]) + extra, dtype=torch.uint8, device="cuda")
+
+
+# --------------------------------------------------------------------------- K2
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", ["fused", "update", "data"])
+def test_compress_matches_oracle(dev, oracle, dtype, mode):
+    rng = np.random.default_rng(11)
+    sizes = [0, 1, 2, 63, 64, 65, 255, 256, 257, 1023, 1024, 4095, 4096, 4097, 8193, 100_003, 1_000_003]
+    for n in sizes:
+        for q in [0.0, 0.9, 0.99, 1.0]:
+            say("compress", dtype.__name__, mode, "n", n, "q", q)
+            d = _rand(rng, n, dtype)
+            u = _rand(rng, n, dtype, 0.5)
+            s = u + d if mode == "fused" else (u if mode == "update" else d)
+            thr = dtype(0) if (q == 0.0 or n == 0) else dtype(np.quantile(np.abs(s), q))
+            dd = d.copy() if mode != "update" else None
+            uu = u.copy() if mode != "data" else None
+            want = oracle.ip_compress(dd, uu, thr)
+            gd = _gpu(d) if mode != "update" else None
+            gu = _gpu(u) if mode != "data" else None
+            buf = _msgbuf(n, dtype)
+            nbytes = dev.compress(buf, gd, gu, thr=thr)
+            assert nbytes == want.size
+            assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+            if uu is not None:
+                assert gu.cpu().numpy().tobytes() == uu.tobytes()
+            if gd is not None:
+                assert gd.cpu().numpy().tobytes() == d.tobytes()  # data is read-only
+    dev.synchronize()
+
+
+@pytest.mark.parametrize("items", [2, 4, 8])
+@pytest.mark.parametrize("tile_ids", [0, 1])
+def test_compress_variants_agree(dev, oracle, items, tile_ids):
+    """Every tile size / tile-order variant of the compaction kernel gives the same bytes."""
+    rng = np.random.default_rng(12)
+    n = 3_000_017
+    d, u = _rand(rng, n, np.float32), _rand(rng, n, np.float32, 0.3)
+    try:
+        dev.set_option("compact_items", items)
+        dev.set_option("compact_tile_ids", tile_ids)
+        for q in [0.0, 0.5, 0.99, 0.9999]:
+            say("variants items", items, "tile_ids", tile_ids, "q", q)
+            thr = np.float32(np.quantile(np.abs(u + d), q)) if q else np.float32(0)
+            uu = u.copy()
+            want = oracle.ip_compress(d.copy(), uu, thr)
+            gu, buf = _gpu(u), _msgbuf(n, np.float32)
+            nbytes = dev.compress(buf, _gpu(d), gu, thr=thr)
+            assert nbytes == want.size
+            assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+            assert gu.cpu().numpy().tobytes() == uu.tobytes()
+    finally:
+        dev.set_option("compact_items", 4)
+        dev.set_option("compact_tile_ids", 0)
+
+
+def test_compress_unaligned_pointers_and_prefix(dev, oracle):
+    """Sub-vectors at odd offsets (ring segments, src/allreduce.tpp:436-437) and the 4-byte
+    sizeBytes prefix (src/comprEx.tpp:184-188) that leaves pairs only 4-byte aligned."""
+    rng = np.random.default_rng(13)
+    n = 50_001
+    for dtype in DTYPES:
+        d, u = _rand(rng, n + 3, dtype), _rand(rng, n + 3, dtype, 0.3)
+        for off in [1, 2, 3]:
+            say("unaligned", dtype.__name__, off)
+            thr = dtype(np.quantile(np.abs(u[off:off + n] + d[off:off + n]), 0.98))
+            uu = u.copy()
+            want = oracle.ip_compress(d[off:off + n].copy(), uu[off:off + n], thr)
+            gd, gu = _gpu(d), _gpu(u)
+            buf = _msgbuf(n, dtype, extra=8)
+            prefix = buf[:4].view(torch.int32)
+            nbytes = dev.compress(buf[4:], gd[off:off + n], gu[off:off + n], thr=thr, size_prefix=prefix)
+            assert nbytes == want.size and int(prefix.item()) == want.size
+            assert buf[4:4 + nbytes].cpu().numpy().tobytes() == want.tobytes()
+            assert gu.cpu().numpy().tobytes() == uu.tobytes()  # elements outside the slice untouched too
+
+
+def test_compress_special_values(dev, oracle):
+    d = np.array([1, np.nan, -3, np.inf, -np.inf, 0.5, -0.0, 0.0] * 700, dtype=np.float32)
+    u = np.zeros_like(d)
+    uu = u.copy()
+    want = oracle.ip_compress(d.copy(), uu, np.float32(0.75))
+    gu, buf = _gpu(u), _msgbuf(d.size, np.float32)
+    nbytes = dev.compress(buf, _gpu(d), gu, thr=0.75)
+    assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+    assert gu.cpu().numpy().tobytes() == uu.tobytes()  # NaN stays in the residual, zeros are +0
+
+
+def test_compress_capacity_and_size_errors(dev):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    d = torch.ones(1000, device="cuda")
+    u = torch.zeros(1000, device="cuda")
+    small = torch.zeros(8 + 8 * 10, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ComprexError) as e:
+        dev.compress(small, d, u, thr=0.5)
+    assert e.value.code == _lib.CX_ERR_CAPACITY
+    assert small[:8].view(torch.int32).tolist() == [1000, 1000]  # header reports the true count
+    with pytest.raises(ComprexError) as e:
+        dev.compress(_msgbuf(1000, np.float32), d, u[:999], thr=0.5)
+    assert e.value.code == _lib.CX_ERR_SIZE_MISMATCH
+    dev.synchronize()  # status is clean again
+
+
+# --------------------------------------------------------------------------- thresholds
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_threshold_matches_oracle(dev, oracle, dtype):
+    rng = np.random.default_rng(14)
+    for n in [1, 2, 5, 999, 1000, 1001, 4096, 50_000, 300_001, 2_000_003]:
+        for topk, ds, sf in [(0.01, 1000, 10.0), (0.1, 1000, 10.0), (0.001, 1000, 10.0), (0.01, 125, 4.0),
+                             (0.02, 1 << 22, 10.0), (1.0, 10, 1.0), (0.5, 1 << 22, 10.0)]:
+            say("threshold", dtype.__name__, n, topk, ds, sf)
+            v, a = _rand(rng, n, dtype), _rand(rng, n, dtype, 0.3)
+            if n > 100:
+                v[rng.integers(0, n, n // 7)] = v[3]  # ties
+            t = np.float32(topk)
+            want_with = oracle.topk_prepare_with(v, a, t, ds, sf)
+            want = oracle.topk_prepare(v, t, ds, sf)
+            gv, ga = _gpu(v), _gpu(a)
+            assert dev.topk_threshold(gv, ga, t, ds, sf) == want_with
+            assert dev.topk_threshold(gv, None, t, ds, sf) == want
+
+
+def test_topk_threshold_indexed_and_device_slot(dev, oracle):
+    rng = np.random.default_rng(15)
+    n, m = 1_000_000, 10_000
+    v, a = _rand(rng, n, np.float32), _rand(rng, n, np.float32, 0.5)
+    idx = rng.integers(0, n, m).astype(np.int32)
+    want = oracle.topk_prepare_indexed(v, a, idx, np.float32(0.01))
+    gv, ga = _gpu(v), _gpu(a)
+    assert dev.topk_threshold_indexed(gv, ga, _gpu(idx), np.float32(0.01)) == want
+    # threshold left on the device and consumed from there by the compressor
+    out = torch.zeros(1, device="cuda")
+    dev.topk_threshold_indexed(gv, ga, _gpu(idx), np.float32(0.01), out=out, to_host=False)
+    buf = _msgbuf(n, np.float32)
+    nbytes = dev.compress(buf, ga, gv, d_thr=out)
+    uu = v.copy()
+    wmsg = oracle.ip_compress(a.copy(), uu, want)
+    assert nbytes == wmsg.size and buf[:nbytes].cpu().numpy().tobytes() == wmsg.tobytes()
+    assert gv.cpu().numpy().tobytes() == uu.tobytes()
+
+
+def test_topk_threshold_errors(dev):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    v = torch.zeros(10, device="cuda")
+    with pytest.raises(ComprexError) as e:
+        dev.topk_threshold(v, torch.zeros(11, device="cuda"), 0.1)
+    assert e.value.code == _lib.CX_ERR_SIZE_MISMATCH
+    for bad in (1.5, -0.1):
+        with pytest.raises(ComprexError) as e:
+            dev.topk_threshold(v, None, bad)
+        assert e.value.code == _lib.CX_ERR_TOPK
+
+
+# --------------------------------------------------------------------------- receive side
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decompress_add_match_oracle(dev, oracle, dtype):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rng = np.random.default_rng(16)
+    for n in [1, 17, 1000, 33_333, 1_000_001]:
+        d = _rand(rng, n, dtype)
+        msg = oracle.ip_compress(d, None, dtype(np.quantile(np.abs(d), 0.9)))
+        gmsg = _gpu(msg)
+        for out_n in [n, n + 13]:
+            say("decompress/add", dtype.__name__, n, out_n)
+            base = _rand(rng, out_n, dtype)
+            o = base.copy()
+            want_bytes = oracle.ip_decompress(msg, o)
+            g = _gpu(base)
+            assert dev.decompress(g, gmsg) == want_bytes
+            assert g.cpu().numpy().tobytes() == o.tobytes()
+            o = base.copy()
+            oracle.ip_add(msg, o)
+            g = _gpu(base)
+            dev.add(g, gmsg)
+            assert g.cpu().numpy().tobytes() == o.tobytes()
+        if n > 1:
+            g = torch.ones(n - 1, dtype=NP2T[dtype], device="cuda")
+            with pytest.raises(ComprexError) as e:
+                dev.decompress(g, gmsg)
+            assert e.value.code == _lib.CX_ERR_MSG_TOO_LARGE and (g == 0).all()
+            g = torch.ones(n - 1, dtype=NP2T[dtype], device="cuda")
+            with pytest.raises(ComprexError) as e:
+                dev.add(g, gmsg)
+            assert e.value.code == _lib.CX_ERR_MSG_TOO_LARGE and (g == 1).all()
+    dev.synchronize()
+
+
+def test_add_duplicate_indices_in_message_order(dev, oracle):
+    rec = np.dtype([("i", np.int32), ("v", np.float32)])
+    body = np.array([(2, 1e8), (2, 1.0), (2, -1e8), (5, 3.0), (7, 1.0), (7, 2.0)], dtype=rec)
+    msg = np.concatenate([np.array([8, 6], np.int32).view(np.uint8), body.view(np.uint8)])
+    want = np.zeros(8, np.float32)
+    oracle.ip_add(msg, want)
+    g = torch.zeros(8, device="cuda")
+    dev.add(g, _gpu(msg))
+    assert g.cpu().numpy().tobytes() == want.tobytes()
+    want = np.ones(8, np.float32)
+    oracle.ip_decompress(msg, want)
+    g = torch.ones(8, device="cuda")
+    dev.decompress(g, _gpu(msg))
+    assert g.cpu().numpy().tobytes() == want.tobytes()
+
+
+def test_index_out_of_range_is_reported_not_written(dev):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rec = np.dtype([("i", np.int32), ("v", np.float32)])
+    body = np.array([(1, 1.0), (99, 5.0), (-4, 5.0)], dtype=rec)
+    msg = np.concatenate([np.array([8, 3], np.int32).view(np.uint8), body.view(np.uint8)])
+    g = torch.zeros(8, device="cuda")
+    dev.add(g, _gpu(msg))
+    with pytest.raises(ComprexError) as e:
+        dev.synchronize()
+    assert e.value.code == _lib.CX_ERR_INDEX
+    assert g.tolist() == [0, 1, 0, 0, 0, 0, 0, 0]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reduce_rank_order_bit_exact_and_atomic_tolerance(dev, oracle, dtype):
+    from comprex_amd import workloads as W
+    n, ranks, k = 1 << 20, 8, 10_000
+    msgs = W.c5_messages(seed=77, n=n, ranks=ranks, k=k, shared=k // 2, dtype=dtype)
+    want = np.zeros(n, dtype)
+    for m in msgs:
+        oracle.ip_add(m, want)
+    gm = [_gpu(m) for m in msgs]
+    for accumulate in (False, True):
+        say("reduce", dtype.__name__, "accumulate", accumulate)
+        base = _rand(np.random.default_rng(5), n, dtype) if accumulate else np.zeros(n, dtype)
+        w = base.copy()
+        for m in msgs:
+            oracle.ip_add(m, w)
+        g = _gpu(base) if accumulate else torch.full((n,), 7, dtype=NP2T[dtype], device="cuda")
+        dev.reduce(g, gm, accumulate=accumulate, mode=0)
+        assert g.cpu().numpy().tobytes() == w.tobytes()
+        # atomics reorder the additions: 1e-6 relative in fp32, 1e-12 in fp64
+        g = _gpu(base) if accumulate else torch.full((n,), 7, dtype=NP2T[dtype], device="cuda")
+        dev.reduce(g, gm, accumulate=accumulate, mode=1)
+        tol = 1e-6 if dtype == np.float32 else 1e-12
+        got = g.cpu().numpy()
+        scale = np.maximum(np.abs(w), 1.0)
+        assert (np.abs(got - w) <= tol * scale * 8).all()
+    dev.synchronize()
+
+
+# --------------------------------------------------------------------------- residual maintenance
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_zero_addvec_apply(dev, oracle, dtype):
+    rng = np.random.default_rng(17)
+    for n in [1, 1000, 100_003]:
+        a, b = _rand(rng, n + 1, dtype), _rand(rng, n + 1, dtype)
+        for off in (0, 1):
+            ga, gb = _gpu(a), _gpu(b)
+            dev.add_vec(ga[off:off + n], gb[off:off + n])
+            w = a.copy()
+            oracle.add_rests(w[off:off + n], np.ascontiguousarray(b[off:off + n]))
+            assert ga.cpu().numpy().tobytes() == w.tobytes()
+            dev.zero(ga[off:off + n])
+            w[off:off + n] = 0
+            assert ga.cpu().numpy().tobytes() == w.tobytes()
+        v = np.ascontiguousarray(a[:n])
+        thr = dtype(np.quantile(np.abs(v), 0.7))
+        hi, lo = dev.threshold_apply(_gpu(v), thr, split=True)
+        whi, wlo = oracle.threshold_apply_split(v, thr)
+        assert hi.cpu().numpy().tobytes() == whi.tobytes() and lo.cpu().numpy().tobytes() == wlo.tobytes()
+        assert dev.threshold_apply(_gpu(v), thr).cpu().numpy().tobytes() == oracle.threshold_apply(v, thr).tobytes()
+
+
+# --------------------------------------------------------------------------- golden fixtures
+def test_small_golden_fixtures(dev):
+    """Outputs of the compiled reference headers, committed under tests/golden/."""
+    import os
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "small_cases.npz"))
+    tags = {"f32": np.float32, "f64": np.float64, "i32": np.int32}
+    keys = sorted({k.rsplit("_grads", 1)[0] for k in z.files if k.endswith("_grads")})
+    assert len(keys) == int(z["n_cases"][0])
+    for key in keys:
+        dtype = tags[key.split("_")[1]]
+        grads = z[key + "_grads"]
+        n, ds = [int(x) for x in z[key + "_params"]]
+        topk = np.float32(z[key + "_topk"][0])
+        say("golden", key, n, topk, ds)
+        rests = torch.zeros(n, dtype=NP2T[dtype], device="cuda")
+        buf = _msgbuf(n, dtype)
+        for it in range(grads.shape[0]):
+            g = _gpu(grads[it])
+            thr = dev.topk_threshold(rests, g, topk, ds, 10.0)
+            assert thr == z[key + "_thr"][it]
+            nbytes = dev.compress(buf, g, rests)  # threshold taken from the handle's device slot
+            want = z["%s_msg%d" % (key, it)]
+            assert nbytes == want.size and buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+            assert rests.cpu().numpy().tobytes() == z["%s_rests%d" % (key, it)].tobytes()
+        g = _gpu(grads[-1])
+        thr = dev.topk_threshold(g, None, topk, ds, 10.0)
+        assert thr == z[key + "_thr_noresidual"][0]
+        want = z[key + "_msg_dataonly"]
+        nbytes = dev.compress(buf, g, None, thr=thr)
+        assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        u = _gpu(grads[-1])
+        want = z[key + "_msg_updateonly"]
+        nbytes = dev.compress(buf, None, u, thr=thr)
+        assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        assert u.cpu().numpy().tobytes() == z[key + "_upd_after"].tobytes()
+        want = z[key + "_msg_flush"]
+        nbytes = dev.compress(buf, rests, None, thr=0)
+        assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        m0 = _gpu(z[key + "_msg0"])
+        o = _gpu(grads[0])
+        dev.decompress(o, m0)
+        assert o.cpu().numpy().tobytes() == z[key + "_dec0"].tobytes()
+        o = _gpu(grads[0])
+        dev.add(o, m0)
+        assert o.cpu().numpy().tobytes() == z[key + "_add0"].tobytes()
