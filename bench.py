@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the compression hot path on one MI355X.
+
+A step = one writeRemote of the 100 M-element workload (config C4): the sampled
+ThresholdTopK threshold from 100 000 host-supplied sample positions (1 % density), then the
+fused accumulate + select + ordered compaction + residual zeroing kernel.  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(g, idx, topk, seconds):
+    """The same step on one host core: the compiled reference headers when their library
+    travelled with the tree, else the plain-C restatement."""
+    from oracle.pyoracle import Oracle, ref_available
+    impl = Oracle(ref=True) if ref_available() else Oracle()
+    n = g.size
+    rests = np.zeros(n, np.float32)
+    times, k = [], 0
+    t_end = time.perf_counter() + seconds
+    it = 0
+    while it < 2 or (time.perf_counter() < t_end and it < 200):
+        t0 = time.perf_counter()
+        sums = rests[idx] + g[idx]                       # prep_add_vec's gather on the chosen positions
+        thr = impl.calc_threshold(sums, topk)            # calc_threshold (nth_element)
+        msg = impl.ip_compress(g, rests, thr)            # compress_add_update
+        dt = time.perf_counter() - t0
+        k = int(msg[4:8].view(np.int32)[0])
+        if it > 0:  # first pass is the warm-up
+            times.append((dt, 12 * n + 8 * k + 8 + 8 * idx.size))
+        it += 1
+    med = sorted(times)[len(times) // 2]
+    return dict(value=med[1] / med[0] / 1e9, unit="GB/s", cores=1, kind=impl.kind,
+                sample="%d full steps (n=%d, %d sample positions) after 1 warm-up, median; %.1f ms/step"
+                       % (len(times), n, idx.size, med[0] * 1e3),
+                ms_per_step=med[0] * 1e3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--n", type=int, default=None, help="override the vector length (debugging)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the exact-top-k and reduce legs")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--items", type=int, default=None, help="compaction tile option (2/4/8)")
+    ap.add_argument("--tile-ids", type=int, default=None, help="0 dynamic tile counter, 1 blockIdx order")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU; the path has no inter-GPU part (--gpus %d refused)" % args.gpus)
+        sys.exit(2)
+
+    import torch
+    from comprex_amd import workloads as W
+    from comprex_amd.device import Handle, message_capacity
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    n = args.n or W.C4["n"]
+    topk = np.float32(W.C4["topK"])
+    m = W.C4["n_samples"] if n >= W.C4["n_samples"] * 10 else max(1000, n // 100)
+
+    t0 = time.time()
+    g_h = W.c4_gradient(n=n)
+    idx_h = W.c4_sample_indices(n=n, m=m)
+    log("generated %s: n=%d in %.1fs (input checksum %s)" % (W.C4["name"], n, time.time() - t0, W.checksum(g_h)))
+
+    h = Handle()
+    if args.items is not None:
+        h.set_option("compact_items", args.items)
+    if args.tile_ids is not None:
+        h.set_option("compact_tile_ids", args.tile_ids)
+    g = torch.from_numpy(g_h).cuda()
+    idx = torch.from_numpy(idx_h).cuda()
+    rests = torch.zeros(n, device="cuda")
+    msg = torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+    hdr = msg[:8].view(torch.int32)
+
+    def step(ev=None):
+        h.topk_threshold_indexed(rests, g, idx, topk, to_host=False)  # threshold stays on the device
+        if ev:
+            ev[0].record()
+        h.compress(msg, g, rests, sync=False)                         # reads it from the handle's slot
+        if ev:
+            ev[1].record()
+
+    for _ in range(args.warmup):
+        step()
+    h.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    h.synchronize()  # raises if any launch recorded a device-side error
+    k = int(hdr[1].item())
+    assert int(hdr[0].item()) == n
+    ms_per_step = elapsed / args.steps * 1e3
+    step_bytes = 12 * n + 8 * k + 8 + 8 * m
+    kern_ms = float(np.mean([a.elapsed_time(b) for a, b in events]))
+    kern_bytes = 12 * n + 8 * k + 8
+    achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
+    log("step %.3f ms, compact kernel %.3f ms (%.0f GB/s, %.1f%% of peak), k=%d (%.3f%%)"
+        % (ms_per_step, kern_ms, achieved, 100 * achieved / HBM_PEAK_GBPS, k, 100.0 * k / n))
+
+    extra = {"k_last_step": k, "density": k / n, "elements_per_s": n / (ms_per_step * 1e-3),
+             "compact_kernel_ms": kern_ms, "threshold_ms": ms_per_step - kern_ms,
+             "hbm_peak_fraction_step": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+    if not args.no_extra:
+        # exact top-k (radix select over all n) + compress, same vector
+        rests.zero_()
+        ds = W.C4["default_subsamples_exact"] if n == W.C4["n"] else 1 << 30
+        for _ in range(2):
+            h.topk_threshold(rests, g, topk, ds, to_host=False)
+            h.compress(msg, g, rests, sync=False)
+        torch.cuda.synchronize()
+        reps = 10
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            h.topk_threshold(rests, g, topk, ds, to_host=False)
+            h.compress(msg, g, rests, sync=False)
+        torch.cuda.synchronize()
+        ex_ms = (time.perf_counter() - t0) / reps * 1e3
+        kx = int(hdr[1].item())
+        extra["exact_topk_step_ms"] = ex_ms
+        extra["exact_topk_GBps"] = (20 * n + 8 * kx + 8) / (ex_ms * 1e-3) / 1e9
+        extra["exact_topk_k"] = kx
+        log("exact top-k step %.3f ms (%.0f GB/s of 20n+8k+8), k=%d" % (ex_ms, extra["exact_topk_GBps"], kx))
+        del g, rests, msg
+        torch.cuda.empty_cache()
+
+        # reduce: 8 simulated ranks' 1 %-dense messages into a 64 Mi dense vector (config C5)
+        c5n = W.C5["n"] if n == W.C4["n"] else 1 << 22
+        c5k = W.C5["k"] if n == W.C4["n"] else c5n // 100
+        t0 = time.time()
+        msgs_h = W.c5_messages(n=c5n, k=c5k, shared=c5k // 2)
+        log("generated %s in %.1fs" % (W.C5["name"], time.time() - t0))
+        msgs = [torch.from_numpy(mm).cuda() for mm in msgs_h]
+        dense = torch.empty(c5n, device="cuda")
+        red_bytes = 4 * c5n + 16 * len(msgs) * c5k
+        for mode, name in ((0, "reduce_ordered"), (1, "reduce_atomic")):
+            for _ in range(2):
+                h.reduce(dense, msgs, accumulate=False, mode=mode)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                h.reduce(dense, msgs, accumulate=False, mode=mode)
+            torch.cuda.synchronize()
+            r_ms = (time.perf_counter() - t0) / reps * 1e3
+            extra[name + "_ms"] = r_ms
+            extra[name + "_GBps"] = red_bytes / (r_ms * 1e-3) / 1e9
+            log("%s %.3f ms (%.0f GB/s of 4n+16Rk)" % (name, r_ms, extra[name + "_GBps"]))
+        h.synchronize()
+
+    cpu = None
+    if not args.no_cpu:
+        t0 = time.time()
+        cpu = cpu_baseline(g_h, idx_h, topk, args.cpu_seconds)
+        log("cpu baseline (%s, 1 core): %.2f GB/s, %.1f ms/step (%.1fs)"
+            % (cpu["kind"], cpu["value"], cpu["ms_per_step"], time.time() - t0))
+
+    out = {
+        "metric": "compress GB/s (algorithmic bytes 12n+8k+8+8m per writeRemote step: sampled top-k threshold + "
+                  "fused accumulate/select/compact/zero), 100M fp32, 1% top-k",
+        "value": step_bytes / (ms_per_step * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": W.C4["name"], "n": n, "topK": float(topk), "sample_positions": m,
+                   "threshold": "sampled ThresholdTopK over host-supplied positions", "input_checksum": W.checksum(g_h)},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "compact_kernel<float,0,4,%d>"
+                     % (args.items or 4), "algorithmic_bytes": kern_bytes, "avg_ms": kern_ms},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -153,12 +153,12 @@ int cx_create(cx_handle* out, void* hip_stream) {
     cx_handle h = new cx_handle_s();
     h->stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e = hipGetDevice(&h->device);
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->tile_counter), 256);
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->redo_flag), 256);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->sel), sizeof(SelectState));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->d_status), 256);
     if (e == hipSuccess) e = hipMalloc(&h->d_thr, 256);
     if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&h->h_pinned), 64, hipHostMallocDefault);
-    if (e == hipSuccess) e = hipMemset(h->tile_counter, 0, 256);
+    if (e == hipSuccess) e = hipMemset(h->redo_flag, 0, 256);
     if (e == hipSuccess) e = hipMemset(h->sel, 0, sizeof(SelectState));
     if (e == hipSuccess) e = hipMemset(h->d_status, 0, 256);
     if (e == hipSuccess) e = hipMemset(h->d_thr, 0, 256);
@@ -173,9 +173,12 @@ int cx_create(cx_handle* out, void* hip_stream) {
 int cx_destroy(cx_handle h) {
     if (!h) return CX_OK;
     (void)hipStreamSynchronize(h->stream);
-    if (h->tile_desc) (void)hipFree(h->tile_desc);
-    if (h->tile_counter) (void)hipFree(h->tile_counter);
+    if (h->staging) (void)hipFree(h->staging);
+    if (h->tile_counts) (void)hipFree(h->tile_counts);
+    if (h->tile_offsets) (void)hipFree(h->tile_offsets);
+    if (h->redo_flag) (void)hipFree(h->redo_flag);
     if (h->sel) (void)hipFree(h->sel);
+    if (h->sel_keys) (void)hipFree(h->sel_keys);
     if (h->d_status) (void)hipFree(h->d_status);
     if (h->d_thr) (void)hipFree(h->d_thr);
     if (h->h_pinned) (void)hipHostFree(h->h_pinned);
@@ -202,9 +205,6 @@ int cx_set_option(cx_handle h, const char* key, int value) {
     if (!strcmp(key, "compact_items")) {
         if (value != 2 && value != 4 && value != 8) return fail(CX_ERR_INVALID, "compact_items must be 2, 4 or 8");
         h->compact_items = value;
-    } else if (!strcmp(key, "compact_tile_ids")) {
-        if (value != 0 && value != 1) return fail(CX_ERR_INVALID, "compact_tile_ids must be 0 or 1");
-        h->compact_tile_ids = value;
     } else if (!strcmp(key, "reduce_variant")) {
         h->reduce_variant = value;
     } else {

@@ -69,21 +69,24 @@ struct cx_handle_s {
     int device = 0;
     hipStream_t stream = nullptr;
 
-    // ordered-compaction scratch: one 64-bit descriptor per tile + the dynamic tile counter
-    unsigned long long* tile_desc = nullptr;
-    size_t tile_desc_cap = 0;          // descriptors allocated
-    unsigned int* tile_counter = nullptr;
-    unsigned int counter_base = 0;     // value of *tile_counter before the next launch
-    unsigned int epoch = 0;            // launch number stamped into descriptors
+    // compaction scratch: per-tile staging slots, counts and final offsets
+    unsigned* staging = nullptr;
+    size_t staging_cap = 0;            // 32-bit words allocated
+    unsigned* tile_counts = nullptr;
+    unsigned* tile_offsets = nullptr;
+    size_t tiles_cap = 0;              // tiles allocated
+    unsigned* redo_flag = nullptr;     // holds the launch number of the last launch that deferred a tile
+    unsigned epoch = 0;                // launch number
 
     cx::SelectState* sel = nullptr;
+    void* sel_keys = nullptr;          // gathered sample keys of the two-launch select
+    size_t sel_keys_bytes = 0;
     cx::DeviceStatus* d_status = nullptr;
     void* d_thr = nullptr;             // 8-byte threshold slot
     int* h_pinned = nullptr;           // 64-byte pinned read-back area
 
     // options
-    int compact_items = 4;             // vector loads per thread and tile
-    int compact_tile_ids = 0;          // 0 = dynamic tile counter, 1 = blockIdx order
+    int compact_items = 4;             // 16-byte loads per lane and tile
     int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
 };
 

@@ -1,24 +1,30 @@
 // Fused error-feedback accumulate + magnitude select + ordered compaction + residual zeroing.
 //
 // Replaces the sequential loop of CompressorIndexPairs<T>::compression_strategy
-// (reference src/compressor.hxx:556-611).  One pass over the vector:
+// (reference src/compressor.hxx:556-611).  Two launches on one stream (three for dense flushes), none of which
+// ever waits on another workgroup (no spin loops, no atomics on the data path):
 //
-//   - each 256-thread block takes one tile of 256*VEC*ITEMS consecutive elements with
-//     16-byte vector loads, lane-contiguous so a wavefront reads 1 KiB per instruction;
-//   - s = update + data (one IEEE add, as the reference's `update[i] += data[i]`),
-//     survivors are |s| > threshold (strict; NaN never survives);
-//   - the rank of a survivor inside the tile comes from wavefront ballots + popcounts,
-//     tile totals are chained across tiles with a decoupled look-back over 64-bit
-//     descriptors {count, launch epoch, state}, so pairs land in ascending index order
-//     exactly as the sequential loop writes them;
-//   - the residual is written back once with survivors replaced by +0.
+//  1. stage_kernel   the HBM-bound pass.  Each wavefront owns one tile of 64*VEC*ITEMS
+//                    consecutive elements, read with 16-byte lane-contiguous loads.
+//                    s = update + data (one IEEE add, as the reference's
+//                    `update[i] += data[i]`), survivors are |s| > threshold (strict, NaN
+//                    never survives).  Ranks inside the tile come from wavefront ballots
+//                    and popcounts, in ascending index order.  Survivors go to the tile's
+//                    private slot of a staging buffer (capacity: 1/8 of the tile), the
+//                    tile's count to counts[tile], and the residual is written back once
+//                    with survivors replaced by +0.  A tile with more survivors than its
+//                    slot holds does nothing but record its count with the "deferred" bit.
+//  2. gather_kernel  each 1024-thread block adds up the counts before its 1024 tiles, scans its
+//                    own, copies its staged slots to their final position in the message with
+//                    lane-contiguous stores (one wavefront per 64 tiles) and processes the few
+//                    deferred tiles it owns straight into their final position, which is known
+//                    by now; the last block writes the header.
+//  3. redo_kernel    launched only when the threshold is known to select (nearly) everything
+//                    (flushRests passes 0): then every tile is deferred, pass 1 was a pure count
+//                    pass, and this kernel does the write pass on the whole GPU.
 //
-// HBM traffic per element (fp32): 4 B data + 4 B residual in, 4 B residual out, plus 8 B
-// per survivor.  No scratch traffic beyond one 8-byte descriptor per tile.
-//
-// Every wait on another tile is bounded: a wave that exhausts its spin budget records
-// CX_ERR_INTERNAL in the status word and carries on with a zero prefix, so the grid
-// always drains.
+// HBM traffic per element at low density (fp32): 4 B data + 4 B residual in, 4 B residual
+// out, plus per survivor 8 B staged + 8 B re-read + 8 B final.
 #include "cx_common.hpp"
 
 namespace cx {
@@ -26,8 +32,9 @@ namespace cx {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kWaves = kBlock / 64;
-constexpr unsigned kSpinLimit = 1u << 22;
+constexpr int kWavesPerBlock = kBlock / 64;
+constexpr unsigned kDeferred = 0x80000000u;
+constexpr int kGatherBlock = 1024;
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -35,116 +42,62 @@ __device__ __forceinline__ float mag(float v) { return fabsf(v); }
 __device__ __forceinline__ double mag(double v) { return fabs(v); }
 __device__ __forceinline__ int mag(int v) { return v < 0 ? -v : v; }
 
-__device__ __forceinline__ unsigned word_of(float v) { return __float_as_uint(v); }
-__device__ __forceinline__ unsigned word_of(int v) { return (unsigned)v; }
-
-// descriptor: [63:32] value | [31:2] epoch | [1:0] state (1 = tile count, 2 = inclusive prefix)
-__device__ __forceinline__ unsigned long long make_desc(unsigned value, unsigned epoch, unsigned state) {
-    return ((unsigned long long)value << 32) | ((unsigned long long)(epoch << 2) | state);
+__device__ __forceinline__ void put_pair(unsigned* w, unsigned index, float v) {
+    w[0] = index;
+    w[1] = __float_as_uint(v);
+}
+__device__ __forceinline__ void put_pair(unsigned* w, unsigned index, int v) {
+    w[0] = index;
+    w[1] = (unsigned)v;
+}
+__device__ __forceinline__ void put_pair(unsigned* w, unsigned index, double v) {
+    const unsigned long long bits = (unsigned long long)__double_as_longlong(v);
+    w[0] = index;
+    w[1] = (unsigned)bits;
+    w[2] = (unsigned)(bits >> 32);
 }
 
-__device__ __forceinline__ unsigned wave_sum(unsigned v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
-// Exclusive prefix of tile `tile`: sum of the counts of tiles [0, tile).  Run by one
-// full wavefront; every lane returns the same value.
-__device__ unsigned look_back(const unsigned long long* desc, unsigned tile, unsigned epoch, int lane,
-                              DeviceStatus* status) {
-    unsigned running = 0;
-    int top = (int)tile - 1;  // nearest predecessor still to be accounted for
-    while (top >= 0) {
-        const int idx = top - lane;  // lane 0 looks at the nearest predecessor
-        unsigned long long d = 0;
-        unsigned spins = 0;
-        bool ready;
-        for (;;) {
-            ready = true;
-            if (idx >= 0) {
-                d = __hip_atomic_load(desc + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const unsigned lo = (unsigned)d;
-                ready = ((lo >> 2) == epoch) && ((lo & 3u) != 0u);
-            }
-            if (__all(ready)) break;
-            if (++spins > kSpinLimit ||
-                ((spins & 1023u) == 0 &&
-                 __hip_atomic_load(&status->code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == CX_ERR_INTERNAL)) {
-                if (lane == 0) atomicCAS(&status->code, 0, (int)CX_ERR_INTERNAL);
-                return running;  // bounded wait expired: give up, the host reports the error
-            }
-            __builtin_amdgcn_s_sleep(1);
-        }
-        const unsigned state = (idx >= 0) ? ((unsigned)d & 3u) : 2u;  // before tile 0: prefix 0
-        const unsigned value = (idx >= 0) ? (unsigned)(d >> 32) : 0u;
-        const unsigned long long has_prefix = __ballot(state == 2u);
-        if (has_prefix != 0ull) {
-            const int first = __ffsll((long long)has_prefix) - 1;  // nearest tile with a full prefix
-            running += wave_sum(lane <= first ? value : 0u);
-            return running;
-        }
-        running += wave_sum(value);
-        top -= 64;
-    }
-    return running;
-}
-
-// MODE 0: update += data, select on update, zero selected   (compress_add_update)
-// MODE 1: select on update, zero selected                    (compress_update)
-// MODE 2: select on data, nothing written back               (compress)
-template <typename T, int MODE, int VEC, int ITEMS>
-__global__ __launch_bounds__(kBlock) void compact_kernel(
-    const T* __restrict__ data, T* __restrict__ update, int n, const T* __restrict__ thr_ptr, T thr_val,
-    unsigned* __restrict__ msg_words, long long cap_pairs, int pairs_aligned8, int* __restrict__ size_prefix,
-    unsigned long long* __restrict__ tile_desc, unsigned* __restrict__ tile_counter, unsigned counter_base,
-    unsigned epoch, unsigned ntiles, int static_tile_ids, DeviceStatus* __restrict__ status) {
-    constexpr int kTile = kBlock * VEC * ITEMS;
-    constexpr int kPairWords = Elem<T>::pair_words;
-
-    __shared__ unsigned s_tile;
-    __shared__ unsigned s_prefix;
-    __shared__ unsigned s_wsum[ITEMS][kWaves];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-
-    unsigned tile;
-    if (static_tile_ids) {
-        tile = blockIdx.x;
-    } else {
-        if (tid == 0) s_tile = atomicAdd(tile_counter, 1u) - counter_base;
-        __syncthreads();
-        tile = s_tile;
-    }
-    if (tile >= ntiles) return;  // cannot happen with a consistent counter; keeps indices in range
-
-    const T thr = thr_ptr ? *thr_ptr : thr_val;
+// One wavefront, one tile.  MODE 0: update += data, select on update, zero selected
+// (compress_add_update); MODE 1: select on update, zero selected (compress_update);
+// MODE 2: select on data, nothing written back (compress).
+// DIRECT false: stage the pairs (or defer the tile); true: write them at `direct_pos`.
+template <typename T, int MODE, int VEC, int ITEMS, bool DIRECT>
+__device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __restrict__ update, long long n,
+                                             T thr, unsigned tile, int lane, unsigned* __restrict__ staging,
+                                             unsigned* __restrict__ counts, unsigned* __restrict__ redo_flag,
+                                             unsigned epoch, unsigned* __restrict__ out_pairs, long long direct_pos,
+                                             long long cap_pairs, DeviceStatus* status) {
+    constexpr int kTile = 64 * VEC * ITEMS;
+    constexpr int kCap = kTile / 8;
+    constexpr int PW = Elem<T>::pair_words;
     const long long base = (long long)tile * kTile;
-    const bool full = base + kTile <= (long long)n;
+    const bool full = base + kTile <= n;
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
 
     T s[ITEMS][VEC];
-    unsigned sel[ITEMS];  // bit c set = element c of load j survives
+    unsigned sel[ITEMS], rank[ITEMS];
+    unsigned total = 0;
+    unsigned valid_mask[ITEMS];
 
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-        const long long e0 = base + (long long)j * (kBlock * VEC) + (long long)tid * VEC;
+        const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
         Pack<T, VEC> u, d;
-        unsigned valid = 0;
+        unsigned valid = (1u << VEC) - 1u;
         if (full) {
             if (MODE != 2) u = *reinterpret_cast<const Pack<T, VEC>*>(update + e0);
             if (MODE != 1) d = *reinterpret_cast<const Pack<T, VEC>*>(data + e0);
-            valid = (1u << VEC) - 1u;
         } else {
+            valid = 0;
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
-                const bool in = e0 + c < (long long)n;
+                const bool in = e0 + c < n;
                 u.x[c] = (MODE != 2 && in) ? update[e0 + c] : (T)0;
                 d.x[c] = (MODE != 1 && in) ? data[e0 + c] : (T)0;
                 valid |= (in ? 1u : 0u) << c;
             }
         }
+        valid_mask[j] = valid;
         unsigned m = 0;
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
@@ -157,132 +110,215 @@ __global__ __launch_bounds__(kBlock) void compact_kernel(
         }
         m &= valid;
         sel[j] = m;
-        if (MODE != 2) {
-            Pack<T, VEC> w;
+        unsigned before = total;
 #pragma unroll
-            for (int c = 0; c < VEC; ++c) w.x[c] = ((m >> c) & 1u) ? (T)0 : s[j][c];
+        for (int c = 0; c < VEC; ++c) {
+            const unsigned long long b = __ballot((m >> c) & 1u);
+            before += __popcll(b & below);
+            total += __popcll(b);
+        }
+        rank[j] = before;  // survivors of this tile that precede this lane's first element of load j
+    }
+
+    unsigned* dst;
+    long long dst_limit;  // pairs that may be written through dst
+    if (DIRECT) {
+        dst = out_pairs + direct_pos * PW;
+        dst_limit = cap_pairs - direct_pos;
+    } else {
+        if (total > (unsigned)kCap) {
+            if (lane == 0) {
+                counts[tile] = total | kDeferred;
+                *redo_flag = epoch;
+            }
+            return;  // no side effects: the redo pass starts from untouched inputs
+        }
+        if (lane == 0) counts[tile] = total;
+        dst = staging + (long long)tile * (kCap * PW);
+        dst_limit = kCap;
+    }
+
+    bool overflow = false;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
+        const unsigned m = sel[j];
+        long long pos = rank[j];
+        Pack<T, VEC> w;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) {
+            const bool keep = (m >> c) & 1u;
+            if (keep) {
+                if (pos < dst_limit) put_pair(dst + pos * PW, (unsigned)(e0 + c), s[j][c]);
+                else overflow = true;
+                ++pos;
+            }
+            w.x[c] = keep ? (T)0 : s[j][c];
+        }
+        if (MODE != 2) {
             if (full) {
                 if (MODE == 0 || m != 0u) *reinterpret_cast<Pack<T, VEC>*>(update + e0) = w;
             } else {
 #pragma unroll
                 for (int c = 0; c < VEC; ++c)
-                    if (((valid >> c) & 1u) && (MODE == 0 || ((m >> c) & 1u))) update[e0 + c] = w.x[c];
+                    if (((valid_mask[j] >> c) & 1u) && (MODE == 0 || ((m >> c) & 1u))) update[e0 + c] = w.x[c];
             }
         }
     }
-
-    // ranks inside each (load j, wavefront): lane-major, then element c
-    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    unsigned rank[ITEMS];
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        unsigned before = 0, total = 0;
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-            const unsigned long long b = __ballot((sel[j] >> c) & 1u);
-            before += __popcll(b & below);
-            total += __popcll(b);
-        }
-        rank[j] = before;
-        if (lane == 0) s_wsum[j][wave] = total;
-    }
-    __syncthreads();
-
-    // offsets of this wavefront's groups inside the tile, order (j, wave)
-    unsigned tile_total = 0;
-    unsigned off[ITEMS];
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-#pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-            if (w == wave) off[j] = tile_total;
-            tile_total += s_wsum[j][w];
-        }
-    }
-
-    if (wave == 0) {
-        unsigned prefix = 0;
-        if (tile == 0) {
-            if (lane == 0)
-                __hip_atomic_store(tile_desc, make_desc(tile_total, epoch, 2u), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-            if (lane == 0)
-                __hip_atomic_store(tile_desc + tile, make_desc(tile_total, epoch, 1u), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-            prefix = look_back(tile_desc, tile, epoch, lane, status);
-            if (lane == 0)
-                __hip_atomic_store(tile_desc + tile, make_desc(prefix + tile_total, epoch, 2u), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        }
-        if (lane == 0) s_prefix = prefix;
-    }
-    __syncthreads();
-    const unsigned prefix = s_prefix;
-
-    unsigned* const pairs = msg_words + 2;
-    bool overflow = false;
-#pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        unsigned m = sel[j];
-        if (m == 0u) continue;
-        long long pos = (long long)prefix + off[j] + rank[j];
-        const long long e0 = base + (long long)j * (kBlock * VEC) + (long long)tid * VEC;
-#pragma unroll
-        for (int c = 0; c < VEC; ++c) {
-            if ((m >> c) & 1u) {
-                if (pos < cap_pairs) {
-                    const unsigned index = (unsigned)(e0 + c);
-                    if constexpr (kPairWords == 2) {
-                        if (pairs_aligned8) {
-                            reinterpret_cast<uint2*>(pairs)[pos] = make_uint2(index, word_of(s[j][c]));
-                        } else {
-                            pairs[2 * pos] = index;
-                            pairs[2 * pos + 1] = word_of(s[j][c]);
-                        }
-                    } else {
-                        const unsigned long long bits = (unsigned long long)__double_as_longlong((double)s[j][c]);
-                        pairs[3 * pos] = index;
-                        pairs[3 * pos + 1] = (unsigned)bits;
-                        pairs[3 * pos + 2] = (unsigned)(bits >> 32);
-                    }
-                } else {
-                    overflow = true;
-                }
-                ++pos;
-            }
-        }
-    }
-    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
-
-    if (tile == ntiles - 1 && tid == 0) {
-        const unsigned k = prefix + tile_total;
-        msg_words[0] = (unsigned)n;
-        msg_words[1] = k;
-        if (size_prefix) *size_prefix = (int)(8u + k * (unsigned)(4 * kPairWords));
-    }
+    if (DIRECT && overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
-void launch_variant(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
-                    long long cap_pairs, int aligned8, int* size_prefix, unsigned ntiles) {
-    hipLaunchKernelGGL((compact_kernel<T, MODE, VEC, ITEMS>), dim3(ntiles), dim3(kBlock), 0, h->stream, data, update, n,
-                       thr_ptr, thr_val, msg_words, cap_pairs, aligned8, size_prefix, h->tile_desc, h->tile_counter,
-                       h->counter_base, h->epoch, ntiles, h->compact_tile_ids, h->d_status);
+__global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
+                                                       const T* __restrict__ thr_ptr, T thr_val,
+                                                       unsigned* __restrict__ staging, unsigned* __restrict__ counts,
+                                                       unsigned* __restrict__ redo_flag, unsigned epoch,
+                                                       unsigned ntiles) {
+    const unsigned tile = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    if (tile >= ntiles) return;
+    const T thr = thr_ptr ? *thr_ptr : thr_val;
+    process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63, staging, counts, redo_flag,
+                                             epoch, nullptr, 0, 0, nullptr);
 }
 
-template <typename T, int VEC, int ITEMS>
-void launch_mode(cx_handle h, int mode, const T* data, T* update, int n, const T* thr_ptr, T thr_val,
-                 unsigned* msg_words, long long cap_pairs, int aligned8, int* size_prefix, unsigned ntiles) {
-    if (mode == 0)
-        launch_variant<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                          size_prefix, ntiles);
-    else if (mode == 1)
-        launch_variant<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                          size_prefix, ntiles);
-    else
-        launch_variant<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                          size_prefix, ntiles);
+template <typename T, int MODE, int VEC, int ITEMS>
+__global__ __launch_bounds__(kBlock) void redo_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
+                                                      const T* __restrict__ thr_ptr, T thr_val,
+                                                      const unsigned* __restrict__ counts,
+                                                      const unsigned* __restrict__ offsets,
+                                                      const unsigned* __restrict__ redo_flag, unsigned epoch,
+                                                      unsigned ntiles, unsigned* __restrict__ out_pairs,
+                                                      long long cap_pairs, DeviceStatus* status) {
+    if (*redo_flag != epoch) return;  // nothing was deferred in this launch
+    const T thr = thr_ptr ? *thr_ptr : thr_val;
+    const unsigned nwaves = gridDim.x * kWavesPerBlock;
+    for (unsigned tile = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6); tile < ntiles; tile += nwaves) {
+        if (!(counts[tile] & kDeferred)) continue;
+        process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, tile, threadIdx.x & 63, nullptr, nullptr, nullptr,
+                                                epoch, out_pairs, (long long)offsets[tile], cap_pairs, status);
+    }
+}
+
+// Final offsets of the tiles and copy of the staged slots to their final place.  A block
+// owns kGatherBlock consecutive tiles: it adds up all counts before them (16-byte loads),
+// scans its own, and each wavefront moves the pairs of its 64 tiles with lane-contiguous
+// stores.  Deferred tiles are either processed here, by the wavefront that owns them
+// (inline_redo), or left to redo_kernel, which then needs offsets[].  The block that owns
+// the last tile writes the message header.
+template <typename T, int MODE, int VEC, int ITEMS>
+__global__ __launch_bounds__(kGatherBlock) void gather_kernel(
+    const T* __restrict__ data, T* __restrict__ update, long long n, const T* __restrict__ thr_ptr, T thr_val,
+    const unsigned* __restrict__ counts, unsigned* __restrict__ offsets, const unsigned* __restrict__ staging,
+    unsigned ntiles, unsigned* __restrict__ msg_words, long long cap_pairs, int* __restrict__ size_prefix,
+    int inline_redo, DeviceStatus* status) {
+    constexpr int PW = Elem<T>::pair_words;
+    constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
+    constexpr int kWaves = kGatherBlock / 64;
+    __shared__ unsigned s_before[kWaves];
+    __shared__ unsigned s_wave_total[kWaves];
+    __shared__ unsigned s_off[kWaves][65];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // pairs emitted by all tiles before this block
+    unsigned before = 0;
+    {
+        const uint4* c4 = reinterpret_cast<const uint4*>(counts);
+        const unsigned nvec = blockIdx.x * (kGatherBlock / 4);
+#pragma unroll 4
+        for (unsigned v = tid; v < nvec; v += kGatherBlock) {
+            const uint4 c = c4[v];
+            before += (c.x & ~kDeferred) + (c.y & ~kDeferred) + (c.z & ~kDeferred) + (c.w & ~kDeferred);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
+    if (lane == 0) s_before[wave] = before;
+
+    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
+    const unsigned tile = first + lane;  // tiles past the end count as empty
+    const unsigned raw = tile < ntiles ? counts[tile] : 0u;
+    const unsigned cnt = raw & ~kDeferred;
+    unsigned incl = cnt;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    unsigned* so = s_off[wave];
+    so[lane] = incl - cnt;
+    const unsigned wave_pairs = __shfl(incl, 63, 64);
+    if (lane == 63) {
+        so[64] = wave_pairs;
+        s_wave_total[wave] = wave_pairs;
+    }
+    const unsigned long long deferred = __ballot((raw & kDeferred) != 0u);
+    __syncthreads();
+    unsigned wave_base = 0;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+        wave_base += s_before[w];
+        if (w < wave) wave_base += s_wave_total[w];
+    }
+    const unsigned tile_off = wave_base + (incl - cnt);
+    if (!inline_redo && tile < ntiles) offsets[tile] = tile_off;
+    if (tile == ntiles - 1) {
+        const unsigned k = tile_off + cnt;
+        msg_words[0] = (unsigned)n;
+        msg_words[1] = k;
+        if (size_prefix) *size_prefix = (int)(8u + k * (unsigned)(4 * PW));
+    }
+
+    unsigned* const pairs = msg_words + 2;
+    bool overflow = false;
+    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * 4) {
+        unsigned src_idx[4];
+        bool live[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const unsigned p = p0 + q * 64 + lane;
+            live[q] = p < wave_pairs;
+            // owner: last tile of this wavefront whose exclusive offset is <= p
+            int lo = 0, hi = 63;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (so[mid] <= p) lo = mid;
+                else hi = mid - 1;
+            }
+            if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
+            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - so[lo]);
+        }
+        unsigned v[4][PW];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (live[q]) {
+#pragma unroll
+                for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
+            }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (live[q]) {
+                const long long dst_pos = (long long)wave_base + p0 + q * 64 + lane;
+                if (dst_pos < cap_pairs) {
+#pragma unroll
+                    for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
+                } else {
+                    overflow = true;
+                }
+            }
+    }
+    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+
+    if (inline_redo && deferred != 0ull) {
+        const T thr = thr_ptr ? *thr_ptr : thr_val;
+        unsigned long long todo = deferred;
+        while (todo) {
+            const int l = __ffsll((long long)todo) - 1;
+            todo &= todo - 1;
+            const unsigned pos = __shfl(tile_off, l, 64);
+            process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, first + l, lane, nullptr, nullptr, nullptr, 0u,
+                                                    pairs, (long long)pos, cap_pairs, status);
+        }
+    }
 }
 
 __global__ void empty_message_kernel(unsigned* msg_words, int n, int* size_prefix) {
@@ -291,19 +327,70 @@ __global__ void empty_message_kernel(unsigned* msg_words, int n, int* size_prefi
     if (size_prefix) *size_prefix = 8;
 }
 
-int ensure_descriptors(cx_handle h, size_t ntiles) {
-    if (ntiles <= h->tile_desc_cap) return CX_OK;
-    size_t cap = h->tile_desc_cap ? h->tile_desc_cap : 4096;
-    while (cap < ntiles) cap *= 2;
-    // the old array may still be read by a kernel in flight on the stream
-    CX_HIP(hipStreamSynchronize(h->stream));
-    if (h->tile_desc) CX_HIP(hipFree(h->tile_desc));
-    h->tile_desc = nullptr;
-    h->tile_desc_cap = 0;
-    CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->tile_desc), cap * sizeof(unsigned long long)));
-    CX_HIP(hipMemsetAsync(h->tile_desc, 0, cap * sizeof(unsigned long long), h->stream));
-    h->tile_desc_cap = cap;
+int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
+    if (ntiles > h->tiles_cap) {
+        size_t cap = h->tiles_cap ? h->tiles_cap : 4096;
+        while (cap < ntiles) cap *= 2;
+        CX_HIP(hipStreamSynchronize(h->stream));  // the old arrays may still be in use
+        if (h->tile_counts) CX_HIP(hipFree(h->tile_counts));
+        if (h->tile_offsets) CX_HIP(hipFree(h->tile_offsets));
+        h->tile_counts = h->tile_offsets = nullptr;
+        h->tiles_cap = 0;
+        CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->tile_counts), cap * sizeof(unsigned)));
+        CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->tile_offsets), cap * sizeof(unsigned)));
+        h->tiles_cap = cap;
+    }
+    if (staging_words > h->staging_cap) {
+        size_t cap = staging_words + staging_words / 8;
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->staging) CX_HIP(hipFree(h->staging));
+        h->staging = nullptr;
+        h->staging_cap = 0;
+        CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->staging), cap * sizeof(unsigned)));
+        h->staging_cap = cap;
+    }
     return CX_OK;
+}
+
+template <typename T, int MODE, int VEC, int ITEMS>
+int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
+               long long cap_pairs, int* size_prefix) {
+    constexpr int kTile = 64 * VEC * ITEMS;
+    constexpr int kCap = kTile / 8;
+    constexpr int PW = Elem<T>::pair_words;
+    const unsigned ntiles = (unsigned)(((long long)n + kTile - 1) / kTile);
+    int rc = ensure_scratch(h, ntiles, (size_t)ntiles * kCap * PW);
+    if (rc != CX_OK) return rc;
+    h->epoch += 1u;
+    if (h->epoch == 0u) h->epoch = 1u;  // 0 is what a fresh flag holds
+    unsigned* redo_flag = h->redo_flag;
+
+    const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
+                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, redo_flag, h->epoch, ntiles);
+    // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
+    // give the second pass the whole GPU instead of the gather kernel's few blocks
+    const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
+    const unsigned gather_blocks = (ntiles + kGatherBlock - 1) / kGatherBlock;
+    hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
+                       update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->tile_offsets, h->staging, ntiles,
+                       msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1, h->d_status);
+    if (dense_hint) {
+        const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
+        hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
+                           update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->tile_offsets, redo_flag, h->epoch,
+                           ntiles, msg_words + 2, cap_pairs, h->d_status);
+    }
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
+template <typename T, int VEC, int ITEMS>
+int launch_mode(cx_handle h, int mode, const T* data, T* update, int n, const T* thr_ptr, T thr_val,
+                unsigned* msg_words, long long cap_pairs, int* size_prefix) {
+    if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
+    if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
+    return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
 }
 
 }  // namespace
@@ -317,52 +404,27 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
         return fail(CX_ERR_INVALID, "compress: message buffer must be 4-byte aligned");
     if (out_capacity < 8) return fail(CX_ERR_CAPACITY, "compress: message buffer smaller than its 8-byte header");
     unsigned* msg_words = static_cast<unsigned*>(out_msg);
-    if (!data && !update) {
-        // the reference falls through all three branches and emits an empty message
+    if ((!data && !update) || n == 0) {
+        // no input vector: the reference falls through all three branches and emits an empty message
         hipLaunchKernelGGL(empty_message_kernel, dim3(1), dim3(1), 0, h->stream, msg_words, n, d_size_prefix);
         CX_HIP(hipGetLastError());
         return CX_OK;
     }
     const int mode = (data && update) ? 0 : (update ? 1 : 2);
     const long long cap_pairs = (out_capacity - 8) / kPairBytes;
-    const int aligned8 = ((reinterpret_cast<uintptr_t>(out_msg) & 7u) == 0) ? 1 : 0;
     const T thr_val = thr_host ? *thr_host : (T)0;
     const T* thr_ptr = thr_host ? nullptr : (d_thr ? d_thr : static_cast<const T*>(h->d_thr));
 
     constexpr int kVec = 16 / (int)sizeof(T);
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(update)) & 15u) == 0;
-    const int items = vec_ok ? h->compact_items : 16;
-    const int vec = vec_ok ? kVec : 1;
-    const long long tile = (long long)kBlock * vec * items;
-    const long long nt = n == 0 ? 1 : ((long long)n + tile - 1) / tile;
-    const unsigned ntiles = (unsigned)nt;
-
-    int rc = ensure_descriptors(h, ntiles);
-    if (rc != CX_OK) return rc;
-    h->epoch = (h->epoch + 1u) & 0x3fffffffu;
-    if (h->epoch == 0u) {  // 30-bit launch counter wrapped: forget every old descriptor
-        CX_HIP(hipMemsetAsync(h->tile_desc, 0, h->tile_desc_cap * sizeof(unsigned long long), h->stream));
-        h->epoch = 1u;
+    if (!vec_ok)  // sub-vectors at odd offsets: scalar loads, same tile order
+        return launch_mode<T, 1, 16>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+    switch (h->compact_items) {
+        case 2: return launch_mode<T, kVec, 2>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+        case 4: return launch_mode<T, kVec, 4>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+        case 8: return launch_mode<T, kVec, 8>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+        default: return fail(CX_ERR_INVALID, "compress: unsupported compact_items %d", h->compact_items);
     }
-
-    if (!vec_ok) {
-        launch_mode<T, 1, 16>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                              d_size_prefix, ntiles);
-    } else if (items == 4) {
-        launch_mode<T, kVec, 4>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                d_size_prefix, ntiles);
-    } else if (items == 8) {
-        launch_mode<T, kVec, 8>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                d_size_prefix, ntiles);
-    } else if (items == 2) {
-        launch_mode<T, kVec, 2>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, aligned8,
-                                d_size_prefix, ntiles);
-    } else {
-        return fail(CX_ERR_INVALID, "compress: unsupported compact_items %d", items);
-    }
-    CX_HIP(hipGetLastError());
-    if (!h->compact_tile_ids) h->counter_base += ntiles;
-    return CX_OK;
 }
 
 template int launch_compact<float>(cx_handle, void*, long long, const float*, float*, int, const float*, const float*, int*);

@@ -20,6 +20,7 @@ namespace cx {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr int kSmallSelect = 1 << 18;  // sample sets up to this size take the two-launch path
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -83,6 +84,7 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
     } else {
         for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
             long long p;
+            bool ok = true;
             if (SMODE == 0) {
                 p = i;
             } else if (SMODE == 1) {
@@ -92,11 +94,12 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
                 if (p < 0) p = 0;
             } else {
                 p = idx[i];
-                if (p < 0 || p >= (long long)n) continue;  // ignore positions outside the vector
+                ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+                if (!ok) p = 0;
             }
             T v = vec[p];
             if (HAS_ADD) v = (T)(v + add[p]);
-            const key_t k = key_of(v);
+            const key_t k = ok ? key_of(v) : (key_t)0;
             if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
         }
     }
@@ -166,6 +169,159 @@ __global__ __launch_bounds__(kBlock) void select_pick_kernel(SelectState* st, in
     }
 }
 
+// ---- small sample sets: two launches ---------------------------------------------------
+// First launch: one thread per sample gathers its key, stores it to `keys` and counts the
+// top digit (LDS histogram merged into the global one).  Second launch, one block: picks the
+// top digit, then finishes the remaining digits over the stored keys with LDS histograms only.
+constexpr int kFinishBlock = 1024;
+
+template <typename T, int SMODE, bool HAS_ADD>
+__global__ __launch_bounds__(kBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                              const int* __restrict__ idx, int m, int n, float stepsize,
+                                                              typename Elem<T>::key_t* __restrict__ keys,
+                                                              SelectState* __restrict__ st, int shift, int bits) {
+    using key_t = typename Elem<T>::key_t;
+    __shared__ unsigned lds_hist[kRadixBins];
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    __syncthreads();
+    const unsigned digit_mask = (1u << bits) - 1u;
+    const int stride = gridDim.x * kBlock;
+    for (int i = blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
+        long long p;
+        bool ok = true;
+        if (SMODE == 0) {
+            p = i;
+        } else if (SMODE == 1) {
+            p = (long long)(int)__fmul_rn((float)i, stepsize);  // (int)(i * stepsize), product in fp32
+            if (p > (long long)n - 1) p = (long long)n - 1;     // the reference would read out of bounds
+            if (p < 0) p = 0;
+        } else {
+            p = idx[i];
+            ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+            if (!ok) p = 0;
+        }
+        T v = vec[p];
+        if (HAS_ADD) v = (T)(v + add[p]);
+        const key_t k = ok ? key_of(v) : (key_t)0;
+        keys[i] = k;
+        atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+        const unsigned c = lds_hist[b];
+        if (c) atomicAdd(&st->hist[b], c);
+    }
+}
+
+// Block-wide: digit holding descending rank `rank` in hist[0..kRadixBins), and how many keys
+// lie above that digit.  All threads get the result.
+__device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long long rank, unsigned long long* s_sum,
+                                           unsigned* s_digit, unsigned long long* s_above, unsigned& digit,
+                                           unsigned long long& above) {
+    constexpr int kPer = kRadixBins / kFinishBlock;  // 2 bins per thread
+    const int t = threadIdx.x;
+    const int hi = kRadixBins - 1 - t * kPer;
+    unsigned cnt[kPer];
+    unsigned long long local = 0;
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        cnt[q] = hist[hi - q];
+        local += cnt[q];
+    }
+    // inclusive scan over threads, top digits first
+    unsigned long long incl = local;
+    const int lane = t & 63, wave = t >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned long long up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) s_sum[wave] = incl;
+    if (t == 0) {
+        *s_digit = 0u;
+        *s_above = 0ull;
+    }
+    __syncthreads();
+    unsigned long long before = incl - local;
+    for (int w = 0; w < wave; ++w) before += s_sum[w];
+    if (rank >= before && rank < before + local) {
+        unsigned long long acc = before;
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            if (rank < acc + cnt[q]) {
+                *s_digit = (unsigned)(hi - q);
+                *s_above = acc;
+                break;
+            }
+            acc += cnt[q];
+        }
+    }
+    __syncthreads();
+    digit = *s_digit;
+    above = *s_above;
+    __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typename Elem<T>::key_t* __restrict__ keys,
+                                                                     int m, SelectState* __restrict__ st,
+                                                                     unsigned long long rank, int plus_one,
+                                                                     T* __restrict__ thr_out) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int kKeyBits = Elem<T>::key_bits;
+    constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
+    __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned long long s_sum[kFinishBlock / 64];
+    __shared__ unsigned s_digit;
+    __shared__ unsigned long long s_above;
+    const int t = threadIdx.x;
+
+    // top digit: counted by the first launch into the global histogram
+    for (int b = t; b < kRadixBins; b += kFinishBlock) {
+        lds_hist[b] = st->hist[b];
+        st->hist[b] = 0u;  // leave it clean for the next run
+    }
+    __syncthreads();
+    key_t prefix = 0, mask = 0;
+    for (int p = 0; p < kPasses; ++p) {
+        int shift = kKeyBits - kRadixBits * (p + 1);
+        int bits = kRadixBits;
+        if (shift < 0) {
+            bits += shift;
+            shift = 0;
+        }
+        if (p > 0) {
+            for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
+            __syncthreads();
+            const unsigned digit_mask = (1u << bits) - 1u;
+            for (int i0 = 0; i0 < m; i0 += kFinishBlock * 8) {
+                key_t kk[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    const int i = i0 + q * kFinishBlock + t;
+                    kk[q] = i < m ? keys[i] : ~prefix;  // a key that cannot match
+                }
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+                    if ((kk[q] & mask) == prefix && i0 + q * kFinishBlock + t < m)
+                        atomicAdd(&lds_hist[(unsigned)(kk[q] >> shift) & digit_mask], 1u);
+            }
+            __syncthreads();
+        }
+        unsigned digit;
+        unsigned long long above;
+        block_pick(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+        prefix |= (key_t)digit << shift;
+        mask |= (key_t)((1ull << bits) - 1ull) << shift;
+        rank -= above;
+    }
+    if (t == 0) {
+        T v = value_of(prefix, T());
+        if (plus_one) v = (T)(v + 1);
+        *thr_out = v;
+    }
+}
+
 template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v; }
 
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
@@ -210,11 +366,45 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
     unsigned long long rank = plus_one ? 0ull : (unsigned long long)pos;
     if (rank > (unsigned long long)(m - 1)) rank = (unsigned long long)(m - 1);
 
-    const bool vec_ok =
-        ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
+    using key_t = typename Elem<T>::key_t;
 
+    if (m <= kSmallSelect) {
+        if ((size_t)m * sizeof(key_t) > h->sel_keys_bytes) {
+            CX_HIP(hipStreamSynchronize(h->stream));
+            if (h->sel_keys) CX_HIP(hipFree(h->sel_keys));
+            h->sel_keys = nullptr;
+            h->sel_keys_bytes = 0;
+            size_t bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
+            CX_HIP(hipMalloc(&h->sel_keys, bytes));
+            h->sel_keys_bytes = bytes;
+        }
+        key_t* keys = static_cast<key_t*>(h->sel_keys);
+        const int shift0 = kKeyBits - kRadixBits;
+        int blocks = (m + kBlock - 1) / kBlock;
+        if (blocks > 2048) blocks = 2048;
+#define CX_FIRST(SM, HA)                                                                                          \
+    hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kBlock), 0, h->stream, vec, add_vec, d_idx, \
+                       m, n, stepsize, keys, h->sel, shift0, kRadixBits)
+        if (add_vec) {
+            if (sample_mode == kSampleFull) CX_FIRST(0, true);
+            else if (sample_mode == kSampleStrided) CX_FIRST(1, true);
+            else CX_FIRST(2, true);
+        } else {
+            if (sample_mode == kSampleFull) CX_FIRST(0, false);
+            else if (sample_mode == kSampleStrided) CX_FIRST(1, false);
+            else CX_FIRST(2, false);
+        }
+#undef CX_FIRST
+        hipLaunchKernelGGL(select_finish_kernel<T>, dim3(1), dim3(kFinishBlock), 0, h->stream, keys, m, h->sel, rank,
+                           plus_one, d_thr_out);
+        CX_HIP(hipGetLastError());
+        return CX_OK;
+    }
+
+    const bool vec_ok =
+        ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
     hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank);
     for (int p = 0; p < kPasses; ++p) {
         int shift = kKeyBits - kRadixBits * (p + 1);

@@ -76,17 +76,16 @@ def test_compress_matches_oracle(dev, oracle, dtype, mode):
 
 
 @pytest.mark.parametrize("items", [2, 4, 8])
-@pytest.mark.parametrize("tile_ids", [0, 1])
-def test_compress_variants_agree(dev, oracle, items, tile_ids):
-    """Every tile size / tile-order variant of the compaction kernel gives the same bytes."""
+def test_compress_variants_agree(dev, oracle, items):
+    """Every tile size of the compaction kernel gives the same bytes, at densities that stage
+    every tile (sparse), defer some (around the 1/8 slot capacity) and defer all (dense)."""
     rng = np.random.default_rng(12)
     n = 3_000_017
     d, u = _rand(rng, n, np.float32), _rand(rng, n, np.float32, 0.3)
     try:
         dev.set_option("compact_items", items)
-        dev.set_option("compact_tile_ids", tile_ids)
-        for q in [0.0, 0.5, 0.99, 0.9999]:
-            say("variants items", items, "tile_ids", tile_ids, "q", q)
+        for q in [0.0, 0.5, 0.85, 0.875, 0.9, 0.99, 0.9999]:
+            say("variants items", items, "q", q)
             thr = np.float32(np.quantile(np.abs(u + d), q)) if q else np.float32(0)
             uu = u.copy()
             want = oracle.ip_compress(d.copy(), uu, thr)
@@ -97,7 +96,25 @@ def test_compress_variants_agree(dev, oracle, items, tile_ids):
             assert gu.cpu().numpy().tobytes() == uu.tobytes()
     finally:
         dev.set_option("compact_items", 4)
-        dev.set_option("compact_tile_ids", 0)
+
+
+def test_compress_clustered_survivors(dev, oracle):
+    """Survivors packed into a few tiles (spikes next to each other) while the rest is empty:
+    dense tiles are deferred and redone, sparse ones staged, in one message."""
+    rng = np.random.default_rng(21)
+    n = 1_000_000
+    for dtype in DTYPES:
+        d = _rand(rng, n, dtype, 0.01) if dtype != np.int32 else rng.integers(-3, 4, n).astype(np.int32)
+        for start in (0, 5000, 123_456, n - 3000):
+            d[start:start + 3000] = dtype(50)
+        d[rng.integers(0, n, 500)] = dtype(-60)
+        u = np.zeros(n, dtype)
+        uu = u.copy()
+        want = oracle.ip_compress(d.copy(), uu, dtype(10))
+        gu, buf = _gpu(u), _msgbuf(n, dtype)
+        nbytes = dev.compress(buf, _gpu(d), gu, thr=dtype(10))
+        assert nbytes == want.size and buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        assert gu.cpu().numpy().tobytes() == uu.tobytes()
 
 
 def test_compress_unaligned_pointers_and_prefix(dev, oracle):
