@@ -6,7 +6,8 @@ import os
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcomprex_gfx950.so")
+# COMPREX_GFX950_LIB selects another build of the same library (e.g. one made with other flags)
+LIB_PATH = os.environ.get("COMPREX_GFX950_LIB") or os.path.join(_HERE, "lib", "libcomprex_gfx950.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 CX_F32, CX_F64, CX_I32 = 0, 1, 2
@@ -47,6 +48,7 @@ def lib():
         "cx_set_stream": (i, [vp, vp]),
         "cx_synchronize": (i, [vp]),
         "cx_set_option": (i, [vp, C.c_char_p, i]),
+        "cx_profile_read": (i, [vp, C.POINTER(C.c_float), i, C.POINTER(i)]),
         "cx_topk_subsamples": (i, [f, i, f]),
         "cx_topk_pos": (i, [C.c_size_t, f]),
         "cx_topk_threshold": (i, [vp, i, vp, vp, i, i, f, i, f, vp, vp]),

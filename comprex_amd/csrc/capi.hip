@@ -182,6 +182,10 @@ int cx_destroy(cx_handle h) {
     if (h->d_status) (void)hipFree(h->d_status);
     if (h->d_thr) (void)hipFree(h->d_thr);
     if (h->h_pinned) (void)hipHostFree(h->h_pinned);
+    if (h->profile_events) {
+        for (int i = 0; i < 2 * cx_handle_s::kProfileRing; ++i) (void)hipEventDestroy(h->profile_events[i]);
+        delete[] h->profile_events;
+    }
     delete h;
     return CX_OK;
 }
@@ -205,11 +209,32 @@ int cx_set_option(cx_handle h, const char* key, int value) {
     if (!strcmp(key, "compact_items")) {
         if (value != 2 && value != 4 && value != 8) return fail(CX_ERR_INVALID, "compact_items must be 2, 4 or 8");
         h->compact_items = value;
+    } else if (!strcmp(key, "profile_stage")) {
+        if (value && !h->profile_events) {
+            h->profile_events = new hipEvent_t[2 * cx_handle_s::kProfileRing];
+            for (int i = 0; i < 2 * cx_handle_s::kProfileRing; ++i) CX_HIP(hipEventCreate(&h->profile_events[i]));
+        }
+        h->profile = value ? 1 : 0;
+        h->profile_count = 0;
+    } else if (!strcmp(key, "stage_alternate")) {
+        h->stage_alternate = value ? 1 : 0;
     } else if (!strcmp(key, "reduce_variant")) {
         h->reduce_variant = value;
     } else {
         return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     }
+    return CX_OK;
+}
+
+int cx_profile_read(cx_handle h, float* ms_out, int max_out, int* n_out) {
+    if (!h || !n_out || (max_out > 0 && !ms_out)) return fail(CX_ERR_INVALID, "cx_profile_read: bad arguments");
+    *n_out = 0;
+    CX_HIP(hipStreamSynchronize(h->stream));
+    const int n = h->profile_count < max_out ? h->profile_count : max_out;
+    for (int i = 0; i < n; ++i)
+        CX_HIP(hipEventElapsedTime(&ms_out[i], h->profile_events[2 * i], h->profile_events[2 * i + 1]));
+    *n_out = n;
+    h->profile_count = 0;
     return CX_OK;
 }
 

@@ -85,8 +85,15 @@ struct cx_handle_s {
     void* d_thr = nullptr;             // 8-byte threshold slot
     int* h_pinned = nullptr;           // 64-byte pinned read-back area
 
+    // optional timing of the streaming pass: HIP events recorded around stage_kernel
+    static constexpr int kProfileRing = 1024;
+    int profile = 0;
+    int profile_count = 0;             // launches recorded since the last read
+    hipEvent_t* profile_events = nullptr;  // 2 * kProfileRing events, created on first use
+
     // options
     int compact_items = 4;             // 16-byte loads per lane and tile
+    int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
     int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
 };
 

@@ -38,6 +38,43 @@ constexpr int kGatherBlock = 1024;
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
+// Cache policy of the streaming pass.  The gradient is read once per step and the residual
+// is rewritten once per step, so both bypass the caches (nontemporal); the residual's READS
+// stay cacheable, which leaves the tail of the pass in the 256 MB memory-side cache, and the
+// next launch walks the tiles in the opposite direction (stage_alternate) to start there.
+#ifndef CX_NT_DATA
+#define CX_NT_DATA 1
+#endif
+#ifndef CX_NT_UPDATE_STORE
+#define CX_NT_UPDATE_STORE 1
+#endif
+
+template <typename T, int V>
+__device__ __forceinline__ Pack<T, V> load_pack(const T* p, bool nt) {
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    Pack<T, V> r;
+    if (nt) {
+        vec_t v = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(p));
+#pragma unroll
+        for (int c = 0; c < V; ++c) r.x[c] = v[c];
+    } else {
+        r = *reinterpret_cast<const Pack<T, V>*>(p);
+    }
+    return r;
+}
+template <typename T, int V>
+__device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& w, bool nt) {
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    if (nt) {
+        vec_t v;
+#pragma unroll
+        for (int c = 0; c < V; ++c) v[c] = w.x[c];
+        __builtin_nontemporal_store(v, reinterpret_cast<vec_t*>(p));
+    } else {
+        *reinterpret_cast<Pack<T, V>*>(p) = w;
+    }
+}
+
 __device__ __forceinline__ float mag(float v) { return fabsf(v); }
 __device__ __forceinline__ double mag(double v) { return fabs(v); }
 __device__ __forceinline__ int mag(int v) { return v < 0 ? -v : v; }
@@ -85,8 +122,8 @@ __device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __re
         Pack<T, VEC> u, d;
         unsigned valid = (1u << VEC) - 1u;
         if (full) {
-            if (MODE != 2) u = *reinterpret_cast<const Pack<T, VEC>*>(update + e0);
-            if (MODE != 1) d = *reinterpret_cast<const Pack<T, VEC>*>(data + e0);
+            if (MODE != 2) u = load_pack<T, VEC>(update + e0, false);
+            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
         } else {
             valid = 0;
 #pragma unroll
@@ -157,7 +194,7 @@ __device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __re
         }
         if (MODE != 2) {
             if (full) {
-                if (MODE == 0 || m != 0u) *reinterpret_cast<Pack<T, VEC>*>(update + e0) = w;
+                if (MODE == 0 || m != 0u) store_pack<T, VEC>(update + e0, w, CX_NT_UPDATE_STORE != 0);
             } else {
 #pragma unroll
                 for (int c = 0; c < VEC; ++c)
@@ -173,9 +210,10 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
                                                        const T* __restrict__ thr_ptr, T thr_val,
                                                        unsigned* __restrict__ staging, unsigned* __restrict__ counts,
                                                        unsigned* __restrict__ redo_flag, unsigned epoch,
-                                                       unsigned ntiles) {
-    const unsigned tile = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+                                                       unsigned ntiles, int reverse) {
+    unsigned tile = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
     if (tile >= ntiles) return;
+    if (reverse) tile = ntiles - 1u - tile;  // start where the previous pass over these vectors ended
     const T thr = thr_ptr ? *thr_ptr : thr_val;
     process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63, staging, counts, redo_flag,
                                              epoch, nullptr, 0, 0, nullptr);
@@ -201,8 +239,8 @@ __global__ __launch_bounds__(kBlock) void redo_kernel(const T* __restrict__ data
 
 // Final offsets of the tiles and copy of the staged slots to their final place.  A block
 // owns kGatherBlock consecutive tiles: it adds up all counts before them (16-byte loads),
-// scans its own, and each wavefront moves the pairs of its 64 tiles with lane-contiguous
-// stores.  Deferred tiles are either processed here, by the wavefront that owns them
+// scans its own, and each lane moves the pairs of its own tile (the first 64 bytes of every
+// slot are fetched before the scan so that the two latencies overlap).  Deferred tiles are either processed here, by the wavefront that owns them
 // (inline_redo), or left to redo_kernel, which then needs offsets[].  The block that owns
 // the last tile writes the message header.
 template <typename T, int MODE, int VEC, int ITEMS>
@@ -216,8 +254,21 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     constexpr int kWaves = kGatherBlock / 64;
     __shared__ unsigned s_before[kWaves];
     __shared__ unsigned s_wave_total[kWaves];
-    __shared__ unsigned s_off[kWaves][65];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
+    const unsigned tile = first + lane;  // tiles past the end count as empty
+    const unsigned raw = tile < ntiles ? counts[tile] : 0u;
+    const unsigned cnt = raw & ~kDeferred;
+    const bool staged = cnt != 0u && !(raw & kDeferred);
+    const unsigned words = staged ? cnt * PW : 0u;  // 32-bit words this lane has to move
+    const uint4* slot = reinterpret_cast<const uint4*>(staging + (long long)tile * (kSlotPairs * PW));
+
+    // first 16 words of the slot are fetched now, so that their latency overlaps the scan below
+    uint4 head[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        if (words > 4u * q) head[q] = slot[q];
 
     // pairs emitted by all tiles before this block
     unsigned before = 0;
@@ -234,23 +285,13 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
     if (lane == 0) s_before[wave] = before;
 
-    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
-    const unsigned tile = first + lane;  // tiles past the end count as empty
-    const unsigned raw = tile < ntiles ? counts[tile] : 0u;
-    const unsigned cnt = raw & ~kDeferred;
     unsigned incl = cnt;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
         const unsigned up = __shfl_up(incl, o, 64);
         if (lane >= o) incl += up;
     }
-    unsigned* so = s_off[wave];
-    so[lane] = incl - cnt;
-    const unsigned wave_pairs = __shfl(incl, 63, 64);
-    if (lane == 63) {
-        so[64] = wave_pairs;
-        s_wave_total[wave] = wave_pairs;
-    }
+    if (lane == 63) s_wave_total[wave] = incl;
     const unsigned long long deferred = __ballot((raw & kDeferred) != 0u);
     __syncthreads();
     unsigned wave_base = 0;
@@ -269,44 +310,36 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     }
 
     unsigned* const pairs = msg_words + 2;
-    bool overflow = false;
-    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * 4) {
-        unsigned src_idx[4];
-        bool live[4];
+    // each lane moves its own tile's pairs; consecutive lanes write consecutive runs
+    if (staged) {
+        long long room = (cap_pairs - (long long)tile_off) * PW;  // words that still fit the message
+        if (room < 0) room = 0;
+        unsigned* dst = pairs + (long long)tile_off * PW;
+        if ((long long)words > room) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+        const unsigned lim = (long long)words < room ? words : (unsigned)room;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const unsigned p = p0 + q * 64 + lane;
-            live[q] = p < wave_pairs;
-            // owner: last tile of this wavefront whose exclusive offset is <= p
-            int lo = 0, hi = 63;
-            while (lo < hi) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (so[mid] <= p) lo = mid;
-                else hi = mid - 1;
-            }
-            if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
-            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - so[lo]);
+            const unsigned w0 = 4u * q;
+            if (w0 < lim) dst[w0] = head[q].x;
+            if (w0 + 1 < lim) dst[w0 + 1] = head[q].y;
+            if (w0 + 2 < lim) dst[w0 + 2] = head[q].z;
+            if (w0 + 3 < lim) dst[w0 + 3] = head[q].w;
         }
-        unsigned v[4][PW];
+        for (unsigned w0 = 16; w0 < lim; w0 += 16) {
+            uint4 more[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-            if (live[q]) {
+            for (int q = 0; q < 4; ++q)
+                if (w0 + 4u * q < words) more[q] = slot[(w0 >> 2) + q];
 #pragma unroll
-                for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
+            for (int q = 0; q < 4; ++q) {
+                const unsigned w = w0 + 4u * q;
+                if (w < lim) dst[w] = more[q].x;
+                if (w + 1 < lim) dst[w + 1] = more[q].y;
+                if (w + 2 < lim) dst[w + 2] = more[q].z;
+                if (w + 3 < lim) dst[w + 3] = more[q].w;
             }
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-            if (live[q]) {
-                const long long dst_pos = (long long)wave_base + p0 + q * 64 + lane;
-                if (dst_pos < cap_pairs) {
-#pragma unroll
-                    for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
-                } else {
-                    overflow = true;
-                }
-            }
+        }
     }
-    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
 
     if (inline_redo && deferred != 0ull) {
         const T thr = thr_ptr ? *thr_ptr : thr_val;
@@ -366,8 +399,16 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     unsigned* redo_flag = h->redo_flag;
 
     const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    hipEvent_t* ev = nullptr;
+    if (h->profile && h->profile_events && h->profile_count < cx_handle_s::kProfileRing) {
+        ev = h->profile_events + 2 * h->profile_count;
+        h->profile_count += 1;
+        CX_HIP(hipEventRecord(ev[0], h->stream));
+    }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
-                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, redo_flag, h->epoch, ntiles);
+                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, redo_flag, h->epoch, ntiles,
+                       (h->stage_alternate && (h->epoch & 1u)) ? 1 : 0);
+    if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
     // give the second pass the whole GPU instead of the gather kernel's few blocks
     const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;

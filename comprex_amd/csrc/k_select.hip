@@ -294,17 +294,29 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
             __syncthreads();
             const unsigned digit_mask = (1u << bits) - 1u;
-            for (int i0 = 0; i0 < m; i0 += kFinishBlock * 8) {
-                key_t kk[8];
+            constexpr int KV = 16 / (int)sizeof(key_t);  // keys per 16-byte load
+            const int nvec = m / KV;
+            const Pack<key_t, KV>* kv = reinterpret_cast<const Pack<key_t, KV>*>(keys);
+            for (int v0 = 0; v0 < nvec; v0 += kFinishBlock * 4) {
+                Pack<key_t, KV> kk[4];
 #pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const int i = i0 + q * kFinishBlock + t;
-                    kk[q] = i < m ? keys[i] : ~prefix;  // a key that cannot match
+                for (int q = 0; q < 4; ++q) {
+                    const int v = v0 + q * kFinishBlock + t;
+                    if (v < nvec) kk[q] = kv[v];
                 }
 #pragma unroll
-                for (int q = 0; q < 8; ++q)
-                    if ((kk[q] & mask) == prefix && i0 + q * kFinishBlock + t < m)
-                        atomicAdd(&lds_hist[(unsigned)(kk[q] >> shift) & digit_mask], 1u);
+                for (int q = 0; q < 4; ++q) {
+                    if (v0 + q * kFinishBlock + t < nvec) {
+#pragma unroll
+                        for (int c = 0; c < KV; ++c)
+                            if ((kk[q].x[c] & mask) == prefix)
+                                atomicAdd(&lds_hist[(unsigned)(kk[q].x[c] >> shift) & digit_mask], 1u);
+                    }
+                }
+            }
+            for (int i = nvec * KV + t; i < m; i += kFinishBlock) {
+                const key_t k1 = keys[i];
+                if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
             }
             __syncthreads();
         }

@@ -59,6 +59,14 @@ class Handle:
     def set_option(self, key, value):
         check(self.lib.cx_set_option(self._h, key.encode(), int(value)))
 
+    def profile_read(self, max_out=1024):
+        """Milliseconds of the streaming kernel of each compress since the last read
+        (needs set_option("profile_stage", 1)); waits for the stream."""
+        buf = (C.c_float * max_out)()
+        n = C.c_int(0)
+        check(self.lib.cx_profile_read(self._h, buf, max_out, C.byref(n)))
+        return [buf[i] for i in range(n.value)]
+
     def synchronize(self):
         """Waits for the stream; raises the first device-side error recorded since the last call."""
         check(self.lib.cx_synchronize(self._h))

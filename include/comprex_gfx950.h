@@ -69,9 +69,17 @@ int cx_set_stream(cx_handle h, void* hip_stream);
 /* Waits for the handle's stream and returns the first device-side error seen since the
  * last call (CX_OK if none), clearing it. */
 int cx_synchronize(cx_handle h);
-/* Tuning switches (compaction tile and ordering variant, reduce variant); see the .md
- * design notes of the source tree.  Unknown keys return CX_ERR_INVALID. */
+/* Tuning switches: "compact_items" (16-byte loads per lane and tile: 2, 4 or 8),
+ * "stage_alternate" (1 = every other compress walks the vector from its end, so that it starts on
+ * what the previous one left in the memory-side cache), "profile_stage" (see cx_profile_read),
+ * "reduce_variant".  Unknown keys return CX_ERR_INVALID. */
 int cx_set_option(cx_handle h, const char* key, int value);
+
+/* No counterpart in the reference: a measurement aid.  After cx_set_option(h, "profile_stage", 1)
+ * every cx_ip_compress records a HIP event before and after its streaming kernel, on the handle's
+ * stream (at most 1024 launches between reads).  This call waits for the stream and returns the
+ * elapsed milliseconds of those launches, oldest first, and forgets them. */
+int cx_profile_read(cx_handle h, float* ms_out, int max_out, int* n_out);
 
 /* ---- thresholds ----------------------------------------------------------- */
 
