@@ -176,6 +176,7 @@ int cx_destroy(cx_handle h) {
     if (h->staging) (void)hipFree(h->staging);
     if (h->tile_counts) (void)hipFree(h->tile_counts);
     if (h->tile_offsets) (void)hipFree(h->tile_offsets);
+    if (h->block_sums) (void)hipFree(h->block_sums);
     if (h->redo_flag) (void)hipFree(h->redo_flag);
     if (h->sel) (void)hipFree(h->sel);
     if (h->sel_keys) (void)hipFree(h->sel_keys);

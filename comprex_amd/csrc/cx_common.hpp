@@ -74,9 +74,11 @@ struct cx_handle_s {
     size_t staging_cap = 0;            // 32-bit words allocated
     unsigned* tile_counts = nullptr;
     unsigned* tile_offsets = nullptr;
+    unsigned* block_sums = nullptr;    // survivors per streaming block
     size_t tiles_cap = 0;              // tiles allocated
     unsigned* redo_flag = nullptr;     // holds the launch number of the last launch that deferred a tile
     unsigned epoch = 0;                // launch number
+    unsigned parity = 0;               // flips every launch: which direction the pass walks
 
     cx::SelectState* sel = nullptr;
     void* sel_keys = nullptr;          // gathered sample keys of the two-launch select

@@ -2,7 +2,7 @@
 //
 // Replaces the sequential loop of CompressorIndexPairs<T>::compression_strategy
 // (reference src/compressor.hxx:556-611).  Two launches on one stream (three for dense flushes), none of which
-// ever waits on another workgroup (no spin loops, no atomics on the data path):
+// ever waits on another workgroup (no spin loops, no global atomics on the data path):
 //
 //  1. stage_kernel   the HBM-bound pass.  Each wavefront owns one tile of 64*VEC*ITEMS
 //                    consecutive elements, read with 16-byte lane-contiguous loads.
@@ -14,8 +14,9 @@
 //                    tile's count to counts[tile], and the residual is written back once
 //                    with survivors replaced by +0.  A tile with more survivors than its
 //                    slot holds does nothing but record its count with the "deferred" bit.
-//  2. gather_kernel  each 1024-thread block adds up the counts before its 1024 tiles, scans its
-//                    own, copies its staged slots to their final position in the message with
+//  2. gather_kernel  each 256-thread block adds up the per-block survivor sums the streaming
+//                    pass left for the tiles before its own 256, scans its own counts,
+//                    copies its staged slots to their final position in the message with
 //                    lane-contiguous stores (one wavefront per 64 tiles) and processes the few
 //                    deferred tiles it owns straight into their final position, which is known
 //                    by now; the last block writes the header.
@@ -31,10 +32,13 @@ namespace cx {
 
 namespace {
 
-constexpr int kBlock = 256;
+#ifndef CX_STAGE_BLOCK
+#define CX_STAGE_BLOCK 256
+#endif
+constexpr int kBlock = CX_STAGE_BLOCK;  // threads of a streaming block: one tile per wavefront
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
-constexpr int kGatherBlock = 1024;
+constexpr int kGatherBlock = 256;  // tiles per gather block = tiles per group sum
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -99,10 +103,11 @@ __device__ __forceinline__ void put_pair(unsigned* w, unsigned index, double v) 
 // MODE 2: select on data, nothing written back (compress).
 // DIRECT false: stage the pairs (or defer the tile); true: write them at `direct_pos`.
 template <typename T, int MODE, int VEC, int ITEMS, bool DIRECT>
-__device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __restrict__ update, long long n,
+__device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* __restrict__ update, long long n,
                                              T thr, unsigned tile, int lane, unsigned* __restrict__ staging,
-                                             unsigned* __restrict__ counts, unsigned* __restrict__ redo_flag,
-                                             unsigned epoch, unsigned* __restrict__ out_pairs, long long direct_pos,
+                                             unsigned* __restrict__ counts,
+                                             unsigned* __restrict__ redo_flag, unsigned epoch,
+                                             unsigned* __restrict__ out_pairs, long long direct_pos,
                                              long long cap_pairs, DeviceStatus* status) {
     constexpr int kTile = 64 * VEC * ITEMS;
     constexpr int kCap = kTile / 8;
@@ -168,7 +173,7 @@ __device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __re
                 counts[tile] = total | kDeferred;
                 *redo_flag = epoch;
             }
-            return;  // no side effects: the redo pass starts from untouched inputs
+            return total;  // no side effects: the redo pass starts from untouched inputs
         }
         if (lane == 0) counts[tile] = total;
         dst = staging + (long long)tile * (kCap * PW);
@@ -203,20 +208,40 @@ __device__ __forceinline__ void process_tile(const T* __restrict__ data, T* __re
         }
     }
     if (DIRECT && overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    return total;
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
 __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
                                                        const T* __restrict__ thr_ptr, T thr_val,
                                                        unsigned* __restrict__ staging, unsigned* __restrict__ counts,
+                                                       unsigned* __restrict__ block_sums,
                                                        unsigned* __restrict__ redo_flag, unsigned epoch,
                                                        unsigned ntiles, int reverse) {
-    unsigned tile = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    // survivors of this block's tiles, summed in LDS; the wavefront that finishes last stores
+    // the sum, which spares the gather kernel a scan over every tile count
+    __shared__ unsigned s_sum, s_done;
+    if (threadIdx.x == 0) {
+        s_sum = 0u;
+        s_done = 0u;
+    }
+    __syncthreads();
+    // reversed launches walk the blocks from the end: they start on what the previous pass left cached
+    const unsigned block = reverse ? gridDim.x - 1u - blockIdx.x : blockIdx.x;
+    const unsigned tile = block * kWavesPerBlock + (threadIdx.x >> 6);
     if (tile >= ntiles) return;
-    if (reverse) tile = ntiles - 1u - tile;  // start where the previous pass over these vectors ended
     const T thr = thr_ptr ? *thr_ptr : thr_val;
-    process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63, staging, counts, redo_flag,
-                                             epoch, nullptr, 0, 0, nullptr);
+    const unsigned total = process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63,
+                                                                    staging, counts, redo_flag, epoch, nullptr, 0, 0,
+                                                                    nullptr);
+    if ((threadIdx.x & 63) == 0) {
+        const unsigned tiles_here = ntiles - block * kWavesPerBlock < (unsigned)kWavesPerBlock
+                                        ? ntiles - block * kWavesPerBlock
+                                        : (unsigned)kWavesPerBlock;
+        atomicAdd(&s_sum, total);  // LDS
+        __threadfence_block();
+        if (atomicAdd(&s_done, 1u) == tiles_here - 1u) block_sums[block] = atomicAdd(&s_sum, 0u);
+    }
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
@@ -238,60 +263,57 @@ __global__ __launch_bounds__(kBlock) void redo_kernel(const T* __restrict__ data
 }
 
 // Final offsets of the tiles and copy of the staged slots to their final place.  A block
-// owns kGatherBlock consecutive tiles: it adds up all counts before them (16-byte loads),
-// scans its own, and each lane moves the pairs of its own tile (the first 64 bytes of every
-// slot are fetched before the scan so that the two latencies overlap).  Deferred tiles are either processed here, by the wavefront that owns them
-// (inline_redo), or left to redo_kernel, which then needs offsets[].  The block that owns
-// the last tile writes the message header.
+// owns kGatherBlock consecutive tiles: it adds up the per-block sums the streaming pass left
+// for the tiles before its own (16-byte loads), scans its own counts, and each wavefront moves the pairs of its 64 tiles
+// with lane-contiguous stores.  Deferred tiles are either processed here, by the wavefront
+// that owns them (inline_redo), or left to redo_kernel, which then needs offsets[].  The
+// block that owns the last tile writes the message header.
 template <typename T, int MODE, int VEC, int ITEMS>
 __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     const T* __restrict__ data, T* __restrict__ update, long long n, const T* __restrict__ thr_ptr, T thr_val,
-    const unsigned* __restrict__ counts, unsigned* __restrict__ offsets, const unsigned* __restrict__ staging,
-    unsigned ntiles, unsigned* __restrict__ msg_words, long long cap_pairs, int* __restrict__ size_prefix,
-    int inline_redo, DeviceStatus* status) {
+    const unsigned* __restrict__ counts, const unsigned* __restrict__ block_sums, unsigned* __restrict__ offsets,
+    const unsigned* __restrict__ staging, unsigned ntiles, unsigned* __restrict__ msg_words, long long cap_pairs,
+    int* __restrict__ size_prefix, int inline_redo, DeviceStatus* status) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
     constexpr int kWaves = kGatherBlock / 64;
     __shared__ unsigned s_before[kWaves];
     __shared__ unsigned s_wave_total[kWaves];
+    __shared__ unsigned s_off[kWaves][65];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
-    const unsigned tile = first + lane;  // tiles past the end count as empty
-    const unsigned raw = tile < ntiles ? counts[tile] : 0u;
-    const unsigned cnt = raw & ~kDeferred;
-    const bool staged = cnt != 0u && !(raw & kDeferred);
-    const unsigned words = staged ? cnt * PW : 0u;  // 32-bit words this lane has to move
-    const uint4* slot = reinterpret_cast<const uint4*>(staging + (long long)tile * (kSlotPairs * PW));
-
-    // first 16 words of the slot are fetched now, so that their latency overlaps the scan below
-    uint4 head[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-        if (words > 4u * q) head[q] = slot[q];
-
-    // pairs emitted by all tiles before this block
     unsigned before = 0;
     {
-        const uint4* c4 = reinterpret_cast<const uint4*>(counts);
-        const unsigned nvec = blockIdx.x * (kGatherBlock / 4);
+        // stage blocks before this block's first tile: kGatherBlock / kWavesPerBlock per gather block
+        const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
+        const unsigned nvec = blockIdx.x * (kGatherBlock / kWavesPerBlock / 4);
 #pragma unroll 4
         for (unsigned v = tid; v < nvec; v += kGatherBlock) {
-            const uint4 c = c4[v];
-            before += (c.x & ~kDeferred) + (c.y & ~kDeferred) + (c.z & ~kDeferred) + (c.w & ~kDeferred);
+            const uint4 c = b4[v];
+            before += c.x + c.y + c.z + c.w;
         }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
     if (lane == 0) s_before[wave] = before;
 
+    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
+    const unsigned tile = first + lane;  // tiles past the end count as empty
+    const unsigned raw = tile < ntiles ? counts[tile] : 0u;
+    const unsigned cnt = raw & ~kDeferred;
     unsigned incl = cnt;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
         const unsigned up = __shfl_up(incl, o, 64);
         if (lane >= o) incl += up;
     }
-    if (lane == 63) s_wave_total[wave] = incl;
+    unsigned* so = s_off[wave];
+    so[lane] = incl - cnt;
+    const unsigned wave_pairs = __shfl(incl, 63, 64);
+    if (lane == 63) {
+        so[64] = wave_pairs;
+        s_wave_total[wave] = wave_pairs;
+    }
     const unsigned long long deferred = __ballot((raw & kDeferred) != 0u);
     __syncthreads();
     unsigned wave_base = 0;
@@ -310,36 +332,44 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     }
 
     unsigned* const pairs = msg_words + 2;
-    // each lane moves its own tile's pairs; consecutive lanes write consecutive runs
-    if (staged) {
-        long long room = (cap_pairs - (long long)tile_off) * PW;  // words that still fit the message
-        if (room < 0) room = 0;
-        unsigned* dst = pairs + (long long)tile_off * PW;
-        if ((long long)words > room) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
-        const unsigned lim = (long long)words < room ? words : (unsigned)room;
+    bool overflow = false;
+    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * 4) {
+        unsigned src_idx[4];
+        bool live[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const unsigned w0 = 4u * q;
-            if (w0 < lim) dst[w0] = head[q].x;
-            if (w0 + 1 < lim) dst[w0 + 1] = head[q].y;
-            if (w0 + 2 < lim) dst[w0 + 2] = head[q].z;
-            if (w0 + 3 < lim) dst[w0 + 3] = head[q].w;
-        }
-        for (unsigned w0 = 16; w0 < lim; w0 += 16) {
-            uint4 more[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                if (w0 + 4u * q < words) more[q] = slot[(w0 >> 2) + q];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const unsigned w = w0 + 4u * q;
-                if (w < lim) dst[w] = more[q].x;
-                if (w + 1 < lim) dst[w + 1] = more[q].y;
-                if (w + 2 < lim) dst[w + 2] = more[q].z;
-                if (w + 3 < lim) dst[w + 3] = more[q].w;
+            const unsigned p = p0 + q * 64 + lane;
+            live[q] = p < wave_pairs;
+            // owner: last tile of this wavefront whose exclusive offset is <= p
+            int lo = 0, hi = 63;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (so[mid] <= p) lo = mid;
+                else hi = mid - 1;
             }
+            if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
+            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - so[lo]);
         }
+        unsigned v[4][PW];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (live[q]) {
+#pragma unroll
+                for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
+            }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (live[q]) {
+                const long long dst_pos = (long long)wave_base + p0 + q * 64 + lane;
+                if (dst_pos < cap_pairs) {
+#pragma unroll
+                    for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
+                } else {
+                    overflow = true;
+                }
+            }
     }
+    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
 
     if (inline_redo && deferred != 0ull) {
         const T thr = thr_ptr ? *thr_ptr : thr_val;
@@ -348,8 +378,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
             const int l = __ffsll((long long)todo) - 1;
             todo &= todo - 1;
             const unsigned pos = __shfl(tile_off, l, 64);
-            process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, first + l, lane, nullptr, nullptr, nullptr, 0u,
-                                                    pairs, (long long)pos, cap_pairs, status);
+            process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, first + l, lane, nullptr, nullptr, nullptr,
+                                                    0u, pairs, (long long)pos, cap_pairs, status);
         }
     }
 }
@@ -371,6 +401,9 @@ int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
         h->tiles_cap = 0;
         CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->tile_counts), cap * sizeof(unsigned)));
         CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->tile_offsets), cap * sizeof(unsigned)));
+        if (h->block_sums) CX_HIP(hipFree(h->block_sums));
+        h->block_sums = nullptr;
+        CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->block_sums), (cap / kWavesPerBlock + 4) * sizeof(unsigned)));
         h->tiles_cap = cap;
     }
     if (staging_words > h->staging_cap) {
@@ -397,6 +430,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     h->epoch += 1u;
     if (h->epoch == 0u) h->epoch = 1u;  // 0 is what a fresh flag holds
     unsigned* redo_flag = h->redo_flag;
+    h->parity ^= 1u;
 
     const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
     hipEvent_t* ev = nullptr;
@@ -406,16 +440,17 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
         CX_HIP(hipEventRecord(ev[0], h->stream));
     }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
-                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, redo_flag, h->epoch, ntiles,
-                       (h->stage_alternate && (h->epoch & 1u)) ? 1 : 0);
+                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, h->block_sums, redo_flag, h->epoch, ntiles,
+                       (h->stage_alternate && h->parity) ? 1 : 0);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
     // give the second pass the whole GPU instead of the gather kernel's few blocks
     const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
     const unsigned gather_blocks = (ntiles + kGatherBlock - 1) / kGatherBlock;
     hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
-                       update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->tile_offsets, h->staging, ntiles,
-                       msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1, h->d_status);
+                       update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->block_sums,
+                       h->tile_offsets, h->staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
+                       h->d_status);
     if (dense_hint) {
         const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
         hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
