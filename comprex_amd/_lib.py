@@ -43,6 +43,9 @@ def lib():
         "cx_abi_version": (i, []),
         "cx_device_count": (i, []),
         "cx_pointer_on_device": (i, [vp]),
+        "cx_device_alloc": (i, [C.POINTER(vp), C.c_size_t]),
+        "cx_device_free": (i, [vp]),
+        "cx_copy": (i, [vp, vp, vp, C.c_size_t]),
         "cx_create": (i, [C.POINTER(vp), vp]),
         "cx_destroy": (i, [vp]),
         "cx_set_stream": (i, [vp, vp]),

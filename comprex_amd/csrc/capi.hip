@@ -146,6 +146,28 @@ int cx_pointer_on_device(const void* p) {
                : 0;
 }
 
+int cx_device_alloc(void** out, size_t bytes) {
+    if (!out) return fail(CX_ERR_INVALID, "cx_device_alloc: null output");
+    *out = nullptr;
+    if (bytes == 0) return CX_OK;
+    CX_HIP(hipMalloc(out, bytes));
+    return CX_OK;
+}
+
+int cx_device_free(void* p) {
+    if (p) CX_HIP(hipFree(p));
+    return CX_OK;
+}
+
+int cx_copy(cx_handle h, void* dst, const void* src, size_t bytes) {
+    if (!h || ((!dst || !src) && bytes > 0)) return fail(CX_ERR_INVALID, "cx_copy: bad arguments");
+    if (bytes == 0) return CX_OK;
+    CX_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, h->stream));
+    // a pageable host buffer may be reused by the caller right away
+    if (!cx_pointer_on_device(dst) || !cx_pointer_on_device(src)) CX_HIP(hipStreamSynchronize(h->stream));
+    return CX_OK;
+}
+
 int cx_create(cx_handle* out, void* hip_stream) {
     if (!out) return fail(CX_ERR_INVALID, "cx_create: null output");
     *out = nullptr;

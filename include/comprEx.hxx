@@ -1,0 +1,451 @@
+// ComprEx<T>: one directed, compressed point-to-point channel with an error-feedback
+// residual, with the public interface of the reference's include/comprEx.hxx:69-166 and the
+// behaviour of src/comprEx.tpp:30-363.  FastComprEx<T> (one-step-stale, double-buffered
+// variant, include/comprEx.hxx:173-227, src/comprEx.tpp:366-514) follows below.
+//
+// What is different from the reference:
+//   * the residual ("rests") lives in device memory, and so do the send/receive buffers;
+//   * the GaspiCxx Source/TargetBuffer pair is replaced by one device buffer per directed
+//     (source, target, tag) triple, owned by the GaspiEnvironment stand-in: the sender's
+//     compressor writes the message where the receiver reads it, ordered by the HIP stream;
+//   * `vector` arguments may be host pointers (staged) or device pointers (used in place);
+//   * a receive with no message pending throws instead of blocking for ever;
+//   * writeRemote only enqueues GPU work; nothing is copied to the host.
+#ifndef COMPREX_H
+#define COMPREX_H
+
+#include <cstdio>
+#include <memory>
+#include <stdexcept>
+#include <vector>
+
+#include "compressor.hxx"
+#include "gaspiEnvironment.hxx"
+#include "threshold.hxx"
+
+template <class VarTYPE>
+class ComprEx {
+protected:
+    std::unique_ptr<Compressor<VarTYPE> > compressor;
+    std::unique_ptr<ThresholdFunction<VarTYPE> > threshold;
+
+    GaspiEnvironment* gaspiCxx_segment;
+
+    // "rests": the error of compression accumulated locally, rests_size elements on the device
+    cxx::DeviceBuffer restsVect;
+    int rests_size;
+    std::vector<VarTYPE> rests_mirror;  // host copy handed out by getRests_p()
+
+    std::shared_ptr<cxx::Channel> srcBuff_data;   // messages this object sends
+    std::shared_ptr<cxx::Channel> targBuff_data;  // messages this object receives
+
+    int srcRank, targRank;
+    int size;              // uncompressed vector length in elements
+    long long bufferSize;  // bytes of the send/receive buffers
+    float size_factor;
+    bool send_sizeBytes;
+
+    cxx::Handle handle_;
+    cxx::DeviceBuffer stage_;
+
+    VarTYPE* rests() const { return static_cast<VarTYPE*>(restsVect.data()); }
+    char* src_address() const { return static_cast<char*>(srcBuff_data->buffer.data()); }
+    char* targ_address() const { return static_cast<char*>(targBuff_data->buffer.data()); }
+
+    void alloc_rests() {
+        restsVect.reserve((size_t)size * sizeof(VarTYPE));
+        rests_size = size;
+        resetRests();
+    }
+
+    // "waitForCompletion" of the reference's TargetBuffer
+    void wait_for_message() {
+        if (targBuff_data->received >= targBuff_data->sent)
+            throw std::runtime_error("Receive issued with no message pending (the reference would block here)!");
+        targBuff_data->received = targBuff_data->sent;
+    }
+
+    // send-side tail shared by all write paths: data-only / update-only / fused compression
+    // of `n` elements into the source buffer at byte offset `at`
+    void compress_into(long long at, const VarTYPE* d_data, VarTYPE* d_update, int n, bool use_threshold) {
+        const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
+        const VarTYPE* d_thr = use_threshold ? threshold->device_threshold() : nullptr;
+        const VarTYPE thr = use_threshold && !d_thr ? threshold->get_threshold() : (VarTYPE)0;
+        compressor->compress_device(src_address() + at + offset, bufferSize - at - offset, d_data, d_update, n, d_thr,
+                                    thr, send_sizeBytes ? reinterpret_cast<int*>(src_address() + at) : nullptr, false);
+    }
+
+public:
+    ComprEx()
+        : compressor(new CompressorNone<VarTYPE>()), threshold(new ThresholdNone<VarTYPE>()), gaspiCxx_segment(NULL),
+          rests_size(0), srcRank(-1), targRank(-1), size(0), bufferSize(0), size_factor(0), send_sizeBytes(false) {}
+
+    ComprEx(GaspiEnvironment* segment, int size, float size_factor = 1.0, bool send_sizeBytes = false)
+        : compressor(new CompressorNone<VarTYPE>()), threshold(new ThresholdNone<VarTYPE>()),
+          gaspiCxx_segment(segment), rests_size(0), srcRank(-1), targRank(-1), size(size), size_factor(size_factor),
+          send_sizeBytes(send_sizeBytes) {
+        // the reference evaluates size*sizeof(T)*size_factor in fp32 and truncates to int; 64 bits here
+        bufferSize = (long long)((float)((size_t)size * sizeof(VarTYPE)) * size_factor);
+    }
+
+    virtual ~ComprEx() {}
+
+    ComprEx(const ComprEx<VarTYPE>& other) : ComprEx() { *this = other; }
+
+    ComprEx<VarTYPE>& operator=(const ComprEx<VarTYPE>& other) {
+        if (srcBuff_data || targBuff_data)
+            throw std::runtime_error("ComprEx object with established connection cannot be assigned to other object!");
+        gaspiCxx_segment = other.gaspiCxx_segment;
+        compressor.reset(other.compressor->clone());
+        threshold.reset(other.threshold->clone());
+        size = other.size;
+        bufferSize = other.bufferSize;
+        size_factor = other.size_factor;
+        send_sizeBytes = other.send_sizeBytes;
+        if (other.rests_size > 0) {  // same length as the other's residual, all zero
+            restsVect.reserve((size_t)other.rests_size * sizeof(VarTYPE));
+            rests_size = other.rests_size;
+            resetRests();
+        } else {
+            rests_size = 0;
+        }
+        return *this;
+    }
+
+    void setCompressor(const Compressor<VarTYPE>& c) { this->compressor.reset(c.clone()); }
+    void setCompressor(const Compressor<VarTYPE>* c) { this->compressor.reset(c->clone()); }
+    void setThreshold(const ThresholdFunction<VarTYPE>& t) { this->threshold.reset(t.clone()); }
+    void setThreshold(const ThresholdFunction<VarTYPE>* t) { this->threshold.reset(t->clone()); }
+
+    void print_rests() {
+        std::vector<VarTYPE> r = getRests();
+        for (size_t it = 0; it < r.size(); ++it) printf("Rests[%d]: %g\n", (int)it, (double)r[it]);
+    }
+
+    virtual void resetRests() {
+        if (rests_size > 0)
+            cxx::check(cx_zero(handle_.get(), cxx::dtype_of<VarTYPE>::value, rests(), rests_size));
+    }
+
+    // Sends the whole residual (no thresholding: every non-zero element) and clears it.
+    virtual void flushRests() {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        compress_into(0, rests(), nullptr, rests_size, false);
+        srcBuff_data->sent += 1;
+        resetRests();
+    }
+
+    std::vector<VarTYPE> getRests() const {
+        std::vector<VarTYPE> out((size_t)rests_size);
+        if (rests_size > 0) {
+            cx_handle h = const_cast<ComprEx<VarTYPE>*>(this)->handle_.get();
+            cxx::check(cx_copy(h, out.data(), rests(), out.size() * sizeof(VarTYPE)));
+            cxx::check(cx_synchronize(h));
+        }
+        return out;
+    }
+
+    void getRests(VarTYPE* data, int size) const {
+        if (size != rests_size) {
+            char error_msg[100];
+            snprintf(error_msg, sizeof error_msg, "Vector of size %d does not match Rests Vector of size %d!\n", size,
+                     rests_size);
+            throw std::runtime_error(error_msg);
+        }
+        cx_handle h = const_cast<ComprEx<VarTYPE>*>(this)->handle_.get();
+        cxx::check(cx_copy(h, data, rests(), (size_t)size * sizeof(VarTYPE)));
+        cxx::check(cx_synchronize(h));
+    }
+
+    void addRests(VarTYPE* data, int size) const {
+        if (size != rests_size) {
+            char error_msg[100];
+            snprintf(error_msg, sizeof error_msg, "Vector of size %d does not match Rests Vector of size %d!\n", size,
+                     rests_size);
+            throw std::runtime_error(error_msg);
+        }
+        ComprEx<VarTYPE>* self = const_cast<ComprEx<VarTYPE>*>(this);
+        cx_handle h = self->handle_.get();
+        cxx::Staged<VarTYPE> d(h, self->stage_, data, (size_t)size, true, true);
+        cxx::check(cx_add_vec(h, cxx::dtype_of<VarTYPE>::value, d.get(), rests(), size));
+        d.flush();
+        cxx::check(cx_synchronize(h));
+    }
+
+    // Host copy of the residual, refreshed by this call (the reference returns a pointer to its
+    // own std::vector; the residual is device memory here).
+    const std::vector<VarTYPE>* getRests_p() {
+        rests_mirror = getRests();
+        return &rests_mirror;
+    }
+    // Device address of the residual (rests_size elements).
+    const VarTYPE* getRests_device() const { return rests(); }
+
+    // residual += vector; entries above the threshold are sent and cleared
+    virtual void writeRemote(const VarTYPE* vector, int size) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cx_handle h = handle_.get();
+        cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
+        threshold->prepare_with(rests(), rests_size, v.get(), size);
+        if (size != rests_size) {
+            char msg[100];
+            snprintf(msg, sizeof msg, "Compressor: Update vector size (%d) is not equal data vector size (%d)!",
+                     rests_size, size);
+            throw std::runtime_error(msg);
+        }
+        compress_into(0, v.get(), rests(), rests_size, true);
+        srcBuff_data->sent += 1;
+    }
+
+    // compression only: no threshold, residual untouched
+    virtual void writeRemote_compressOnly(const VarTYPE* vector, int size) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cx_handle h = handle_.get();
+        cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
+        compress_into(0, v.get(), nullptr, size, false);
+        srcBuff_data->sent += 1;
+    }
+
+    // threshold from the vector alone, residual untouched
+    void writeRemote_NoResidual(const VarTYPE* vector, int size) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cx_handle h = handle_.get();
+        cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
+        threshold->prepare(v.get(), size);
+        compress_into(0, v.get(), nullptr, size, true);
+        srcBuff_data->sent += 1;
+    }
+
+    // overwrites `vector` with the received message
+    virtual void readRemote(VarTYPE* vector, int size) {
+        if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
+        wait_for_message();
+        const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
+        compressor->decompress(vector, size, targ_address() + offset);
+    }
+
+    // adds the received message to `vector`
+    virtual void readRemote_add(VarTYPE* vector, int size) {
+        if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
+        wait_for_message();
+        const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
+        compressor->add(vector, size, targ_address() + offset);
+    }
+
+    // receive, pass the compressed message on to this object's target, and decompress it
+    void readRemote_forward(VarTYPE* vector, int size) {
+        wait_for_message();
+        cx_handle h = handle_.get();
+        if (send_sizeBytes) {
+            int sizeBytes = 0;
+            cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
+            cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
+            srcBuff_data->sent += 1;
+            compressor->decompress(vector, size, targ_address() + sizeof(int));
+        } else {
+            const int sizeBytes = compressor->decompress(vector, size, targ_address());
+            cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes));
+            srcBuff_data->sent += 1;
+        }
+    }
+
+    void readRemote_forwardCopy(VarTYPE* vector, int size) {
+        if (!this->send_sizeBytes)
+            throw std::runtime_error("If using readRemote_forwardCopy, send_sizeBytes must be true!");
+        wait_for_message();
+        cx_handle h = handle_.get();
+        int sizeBytes = 0;
+        cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
+        cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
+    }
+
+    void readRemote_wait() { wait_for_message(); }
+
+    void forward_buffer() {
+        if (!this->send_sizeBytes) throw std::runtime_error("If using forward_buffer, send_sizeBytes must be true!");
+        cx_handle h = handle_.get();
+        int sizeBytes = 0;
+        cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
+        cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
+    }
+
+    void forward_add(VarTYPE* vector, int size) {
+        if (!this->send_sizeBytes) throw std::runtime_error("If using forward_add, send_sizeBytes must be true!");
+        srcBuff_data->sent += 1;
+        compressor->add(vector, size, src_address() + sizeof(int));
+    }
+
+    virtual void connectTx(int targRank, int tag) {
+        this->targRank = targRank;
+        alloc_rests();  // the residual exists only on objects that send
+        srcBuff_data = gaspiCxx_segment->channel(gaspiCxx_segment->get_rank(), targRank, tag, bufferSize);
+        srcBuff_data->has_sender = true;
+    }
+
+    virtual void connectRx(int srcRank, int tag) {
+        this->srcRank = srcRank;
+        targBuff_data = gaspiCxx_segment->channel(srcRank, gaspiCxx_segment->get_rank(), tag, bufferSize);
+        targBuff_data->has_receiver = true;
+    }
+
+    // srcRank: receive data from this rank; targRank: send data to this rank
+    virtual void connectTo(int srcRank, int targRank, int tag) {
+        connectTx(targRank, tag);
+        connectRx(srcRank, tag);
+    }
+};
+
+// ---------------------------------------------------------------------------------------
+// FastComprEx: the message compressed by one writeRemote is sent by the NEXT one (the
+// reference overlaps the RDMA put of message i-1 with the compression of message i); the
+// source buffer is split in two halves used alternately.
+template <class VarTYPE>
+class FastComprEx : public ComprEx<VarTYPE> {
+protected:
+    int doublebuffer_phase;
+    long long doublebuffer_offset;  // bytes between the two halves
+    bool is_first;
+    // the half that holds the message of the previous call is what the receiver sees: it is
+    // copied to the front of the channel when it is "sent"
+    cxx::DeviceBuffer halves_;
+
+    using ComprEx<VarTYPE>::restsVect;
+    using ComprEx<VarTYPE>::srcBuff_data;
+
+    long long send_offset() const { return doublebuffer_offset * ((doublebuffer_phase + 1) % 2); }
+    long long write_offset() const { return doublebuffer_offset * doublebuffer_phase; }
+    void update_doublebuffer_phase() { doublebuffer_phase = (doublebuffer_phase + 1) % 2; }
+    char* half(long long off) const { return static_cast<char*>(halves_.data()) + off; }
+
+    void ensure_halves() {
+        if (!halves_.data()) halves_.reserve((size_t)(2 * doublebuffer_offset > 32 ? 2 * doublebuffer_offset : 32));
+    }
+
+    // "initTransferPart(sizeBytes, send_offset)": hand the half at `off` to the receiver
+    void send_half(long long off) {
+        cx_handle h = this->handle_.get();
+        // the message's own header tells its length; copy header first, then the pairs it announces
+        int hdr[2] = {0, 0};
+        cxx::check(cx_copy(h, hdr, half(off), 8));
+        const size_t bytes = 8 + (size_t)(hdr[1] < 0 ? 0 : hdr[1]) * (4 + sizeof(VarTYPE));
+        cxx::check(cx_copy(h, this->src_address(), half(off), bytes));
+        srcBuff_data->sent += 1;
+    }
+
+    void compress_half(long long off, const VarTYPE* d_data, VarTYPE* d_update, int n, bool use_threshold) {
+        const VarTYPE* d_thr = use_threshold ? this->threshold->device_threshold() : nullptr;
+        const VarTYPE thr = use_threshold && !d_thr ? this->threshold->get_threshold() : (VarTYPE)0;
+        this->compressor->compress_device(half(off), doublebuffer_offset, d_data, d_update, n, d_thr, thr, nullptr,
+                                          false);
+    }
+
+public:
+    FastComprEx() : ComprEx<VarTYPE>(), doublebuffer_phase(0), doublebuffer_offset(0), is_first(true) {}
+
+    FastComprEx(GaspiEnvironment* segment, int size, float size_factor = 1.0)
+        : ComprEx<VarTYPE>(segment, size, size_factor * 2), doublebuffer_phase(0), is_first(true) {
+        doublebuffer_offset = (long long)((float)size * size_factor * (float)sizeof(VarTYPE));
+    }
+
+    FastComprEx(const FastComprEx<VarTYPE>& other) : ComprEx<VarTYPE>() { *this = other; }
+
+    FastComprEx<VarTYPE>& operator=(const FastComprEx<VarTYPE>& other) {
+        ComprEx<VarTYPE>::operator=(other);
+        doublebuffer_offset = other.doublebuffer_offset;
+        doublebuffer_phase = 0;
+        is_first = true;
+        return *this;
+    }
+
+    virtual void flushRests() {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        ensure_halves();
+        const long long so = send_offset();
+        if (is_first) {
+            // nothing compressed yet: the half is undefined in the reference (it adds whatever the
+            // buffer holds); an empty message is what a fresh buffer of zeros decodes to
+            compress_half(so, nullptr, nullptr, this->rests_size, false);
+        }
+        // the message that was compressed but never sent goes back into the residual ...
+        this->compressor->add_device(this->rests(), this->rests_size, half(so));
+        // ... and the whole residual is sent
+        compress_half(so, this->rests(), nullptr, this->rests_size, false);
+        send_half(so);
+        ComprEx<VarTYPE>::resetRests();
+        is_first = true;
+    }
+
+    virtual void resetRests() {
+        ComprEx<VarTYPE>::resetRests();
+        is_first = true;
+    }
+
+    virtual void writeRemote(const VarTYPE* vector, int size) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        ensure_halves();
+        cx_handle h = this->handle_.get();
+        const long long wo = write_offset(), so = send_offset();
+        if (is_first) {
+            // the residual is all zero at this point, so this is an (almost) empty message
+            compress_half(so, nullptr, this->rests(), this->rests_size, true);
+            is_first = false;
+        }
+        send_half(so);  // the message of the previous call
+        cxx::Staged<const VarTYPE> v(h, this->stage_, vector, (size_t)size, true, false);
+        this->threshold->prepare_with(this->rests(), this->rests_size, v.get(), size);
+        if (size != this->rests_size) {
+            char msg[100];
+            snprintf(msg, sizeof msg, "Compressor: Update vector size (%d) is not equal data vector size (%d)!",
+                     this->rests_size, size);
+            throw std::runtime_error(msg);
+        }
+        compress_half(wo, v.get(), this->rests(), this->rests_size, true);
+        update_doublebuffer_phase();
+    }
+
+    virtual void writeRemote_compressOnly(VarTYPE* vector, int size) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        ensure_halves();
+        cx_handle h = this->handle_.get();
+        const long long wo = write_offset(), so = send_offset();
+        if (is_first) {
+            compress_half(so, this->rests(), nullptr, this->rests_size, false);
+            is_first = false;
+        }
+        send_half(so);
+        cxx::Staged<const VarTYPE> v(h, this->stage_, vector, (size_t)size, true, false);
+        compress_half(wo, v.get(), nullptr, size, false);
+        update_doublebuffer_phase();
+    }
+
+    // Sends what `other` compressed, without compressing again (the chief's broadcast to the
+    // second and later workers, reference src/allreduce.tpp:209).
+    virtual void writeRemote_sameAs(const FastComprEx* other) {
+        if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        ensure_halves();
+        const_cast<FastComprEx*>(other)->ensure_halves();
+        cx_handle h = this->handle_.get();
+        const long long wo = write_offset(), so = send_offset();
+        if (is_first) {
+            compress_half(so, nullptr, this->rests(), this->rests_size, true);
+            is_first = false;
+        }
+        send_half(so);
+        if (!other->is_first) {
+            int hdr[2] = {0, 0};
+            cxx::check(cx_copy(h, hdr, other->half(other->send_offset()), 8));
+            const size_t bytes = 8 + (size_t)(hdr[1] < 0 ? 0 : hdr[1]) * (4 + sizeof(VarTYPE));
+            cxx::check(cx_copy(h, half(wo), other->half(other->send_offset()), bytes));
+        } else {
+            this->is_first = true;
+        }
+        update_doublebuffer_phase();
+    }
+
+    virtual void connectTx_sameBufferAs(int targRank, int tag, const FastComprEx<VarTYPE>* other) {
+        if (!other->srcBuff_data) throw std::runtime_error("Cannot connected with buffer of unconnected communicator!");
+        this->connectTx(targRank, tag);
+    }
+};
+
+#endif  // COMPREX_H

@@ -59,6 +59,14 @@ int cx_device_count(void);
 /* 1 when `p` is device (or managed/host-registered) memory, 0 for pageable host memory. */
 int cx_pointer_on_device(const void* p);
 
+/* Device memory for callers without a HIP runtime of their own (the C++ classes of this
+ * library's headers keep the residual and their staging buffers in it).  cx_copy moves bytes
+ * between any two pointers (host or device) in stream order and waits when a pageable host
+ * buffer is involved.  They stand in for the std::vector / memcpy of src/comprEx.tpp:149-157. */
+int cx_device_alloc(void** out, size_t bytes);
+int cx_device_free(void* p);
+int cx_copy(cx_handle h, void* dst, const void* src, size_t bytes);
+
 /* A handle owns one HIP stream reference and the scratch memory of one compressor
  * clone (tile descriptors, histograms, a device-side threshold slot, a status word).
  * It replaces the per-object state of Compressor<T>/ThresholdFunction<T> clones
@@ -191,6 +199,8 @@ float ThresholdConst_getThreshold(void* self);
 void* ThresholdTopK_new(float topK);
 void ThresholdTopK_del(void* self);
 float ThresholdTopK_getThreshold(void* self);
+void* CompressorNone_new(void);
+void CompressorNone_del(void* self);
 void* CompressorIndexPairs_new(void);
 void CompressorIndexPairs_del(void* self);
 /* Error text of the last reference-ABI call that failed on this thread ("" if none).  The

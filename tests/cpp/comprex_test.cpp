@@ -1,0 +1,158 @@
+// Mirrors the reference's integration tests with simulated ranks in one process:
+//   test/comprex.cpp           2 ranks, 3 x writeRemote + flushRests, gold (num_runs-1)*values
+//   test/AllToOneAllreduce.cpp R ranks, chief reduces in rank order then broadcasts,
+//                              gold (num_runs*(numRanks-1)+1)*values at the chief after flush
+// The rank a call acts as is chosen with GaspiEnvironment::set_rank (the reference gets it from
+// gaspi_run).
+#include <comprEx.hxx>
+
+#include <map>
+#include <vector>
+
+#include "common.hxx"
+
+template <typename data_t> int comprex_p2p(const char* name) {
+    const int size = 50;
+    const int num_runs = 4;
+    const int size_factor = 3;
+    const float threshold = 0.1;
+    std::vector<data_t> values(size), gold_result(size), result(size, (data_t)0);
+    for (int i = 0; i < size; ++i) values[i] = (data_t)(i * (1 - 2 * (i % 2)));
+    for (int i = 0; i < size; ++i) gold_result[i] = (data_t)((num_runs - 1) * values[i]);
+
+    GaspiEnvironment env(1 << 28);
+    const int tag = 1;
+    std::vector<ComprEx<data_t> > cmprex;  // index = rank
+    cmprex.reserve(2);
+    for (int rank = 0; rank < 2; ++rank) {
+        env.set_rank(rank, 2);
+        cmprex.emplace_back(env.get_segment(), size, size_factor, true);
+        cmprex[rank].setThreshold(ThresholdTopK<data_t>(threshold));
+        cmprex[rank].setCompressor(CompressorIndexPairs<data_t>());
+        cmprex[rank].connectTo((rank + 1) % 2, (rank + 1) % 2, tag);
+    }
+    for (int run = 0; run < num_runs; ++run) {
+        if (run < num_runs - 1) cmprex[0].writeRemote(values.data(), (int)values.size());
+        else cmprex[0].flushRests();
+        cmprex[1].readRemote_add(result.data(), (int)result.size());
+    }
+    int errors = 0;
+    for (int i = 0; i < size; ++i)
+        if (result[i] != gold_result[i]) {
+            std::cout << "Error in [" << i << "]: result: " << result[i] << " gold: " << gold_result[i] << std::endl;
+            ++errors;
+        }
+    std::vector<data_t> rests = cmprex[0].getRests();
+    for (auto e : rests) if (e != 0) ++errors;
+    std::cout << "ComprEx point to point (" << name << ")" << std::endl;
+    return print_pass(errors);
+}
+
+// Comprex_AllToOneAllreduce::apply / flush (reference src/allreduce.tpp:172-237), every rank's
+// part executed in the order the data dependencies impose.
+template <typename data_t> int all_to_one(const char* name, int numRanks, int size, int num_runs, float ratio) {
+    const int chief = 0, tag = 1;
+    const int comprexTag = tag * 2 * numRanks, commTag = tag * 2 * numRanks + 1;
+    std::vector<data_t> values(size), gold(size);
+    for (int i = 0; i < size; ++i) values[i] = (data_t)((i % 97) * (1 - 2 * (i % 2)));
+    for (int i = 0; i < size; ++i) gold[i] = (data_t)((num_runs * (numRanks - 1) + 1) * values[i]);
+
+    GaspiEnvironment env(1 << 28);
+    FastComprEx<data_t> proto(env.get_segment(), size, 3.0f);
+    proto.setThreshold(ThresholdTopK<data_t>(ratio));
+    proto.setCompressor(CompressorIndexPairs<data_t>());
+    // per rank: its reduce and broadcast communicators, keyed by peer (src/allreduce.tpp:147-170)
+    std::vector<std::map<int, FastComprEx<data_t> > > reduce(numRanks), bcast(numRanks);
+    for (int rank = 0; rank < numRanks; ++rank) {
+        env.set_rank(rank, numRanks);
+        if (rank == chief) {
+            for (int r = 0; r < numRanks; ++r) {
+                if (r == chief) continue;
+                reduce[rank][r] = proto;
+                reduce[rank][r].connectRx(r, comprexTag + r);
+                bcast[rank][r] = proto;
+                bcast[rank][r].connectTx(r, commTag + r);
+            }
+        } else {
+            reduce[rank][chief] = proto;
+            reduce[rank][chief].connectTx(chief, comprexTag + rank);
+            bcast[rank][chief] = proto;
+            bcast[rank][chief].connectRx(chief, commTag + rank);
+        }
+    }
+    // test/AllToOneAllreduce.cpp:72-90: the chief's vector accumulates over the runs, the workers
+    // start every run from `values`
+    std::vector<std::vector<data_t> > result(numRanks, values);
+    for (int run = 0; run < num_runs; ++run) {
+        for (int rank = 0; rank < numRanks; ++rank)
+            if (rank != chief) result[rank] = values;
+        // apply(), workers' first half: send own data
+        for (int rank = 0; rank < numRanks; ++rank)
+            if (rank != chief) reduce[rank][chief].writeRemote(result[rank].data(), size);
+        // apply(), chief: reduce in ascending rank order ...
+        for (int r = 0; r < numRanks; ++r)
+            if (r != chief) reduce[chief][r].readRemote_add(result[chief].data(), size);
+        // ... and broadcast: compress once, re-send the same buffer to the others
+        int copy_rank = -1;
+        for (int r = 0; r < numRanks; ++r) {
+            if (r == chief) continue;
+            if (copy_rank == -1) { bcast[chief][r].writeRemote(result[chief].data(), size); copy_rank = r; }
+            else bcast[chief][r].writeRemote_sameAs(&bcast[chief][copy_rank]);
+        }
+        // apply(), workers' second half: receive the broadcast
+        for (int rank = 0; rank < numRanks; ++rank)
+            if (rank != chief) bcast[rank][chief].readRemote(result[rank].data(), size);
+    }
+    // flush(): workers send their residuals, the chief adds them; no broadcast; everything is reset
+    for (int rank = 0; rank < numRanks; ++rank)
+        if (rank != chief) reduce[rank][chief].flushRests();
+    for (int r = 0; r < numRanks; ++r)
+        if (r != chief) reduce[chief][r].readRemote_add(result[chief].data(), size);
+    for (int rank = 0; rank < numRanks; ++rank) {
+        for (auto& c : reduce[rank]) c.second.resetRests();
+        for (auto& c : bcast[rank]) c.second.resetRests();
+    }
+    const std::vector<data_t>& total = result[chief];
+    int errors = 0;
+    for (int i = 0; i < size; ++i)
+        if (total[i] != gold[i]) {
+            if (errors < 5) std::cout << "Error in [" << i << "]: result: " << total[i] << " gold: " << gold[i] << std::endl;
+            ++errors;
+        }
+    std::cout << "All-to-one allreduce over " << numRanks << " simulated ranks (" << name << ", n=" << size << ")" << std::endl;
+    return print_pass(errors);
+}
+
+int error_paths() {
+    int errors = 0;
+    GaspiEnvironment env(1 << 20);
+    env.set_rank(0, 2);
+    ComprEx<float> c(env.get_segment(), 16);
+    std::vector<float> v(16, 1.0f);
+    try { c.writeRemote(v.data(), 16); ++errors; } catch (const std::runtime_error&) {}   // not connected
+    try { c.readRemote(v.data(), 16); ++errors; } catch (const std::runtime_error&) {}
+    try { c.flushRests(); ++errors; } catch (const std::runtime_error&) {}
+    c.setThreshold(ThresholdTopK<float>(0.5f));
+    c.setCompressor(CompressorIndexPairs<float>());
+    c.connectTo(1, 1, 7);
+    try { c.writeRemote(v.data(), 15); ++errors; } catch (const std::runtime_error&) {}   // size mismatch
+    try { c.getRests(v.data(), 15); ++errors; } catch (const std::runtime_error&) {}
+    try { c.addRests(v.data(), 15); ++errors; } catch (const std::runtime_error&) {}
+    try { c.readRemote(v.data(), 16); ++errors; } catch (const std::runtime_error&) {}    // nothing pending
+    ComprEx<float> d(env.get_segment(), 16);
+    try { c = d; ++errors; } catch (const std::runtime_error&) {}                          // connected object
+    std::cout << "ComprEx error paths" << std::endl;
+    return print_pass(errors);
+}
+
+int main() {
+    if (!need_gpu()) return 77;
+    int failed = 0;
+    failed += comprex_p2p<int>("int");
+    failed += comprex_p2p<float>("float");
+    failed += comprex_p2p<double>("double");
+    failed += all_to_one<int>("int", 4, 1000, 10, 0.01f);
+    failed += all_to_one<float>("float", 3, 100000, 5, 0.001f);
+    failed += error_paths();
+    return failed ? 1 : 0;
+}

@@ -1,0 +1,148 @@
+"""The drop-in layers above the kernels, on the GPU: the C++ classes (driven by C++ tests that
+mirror the reference's own) and the reference's float C ABI behind its Python wrappers."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.pyoracle import parse_message
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin")
+
+
+@pytest.mark.parametrize("name", ["threshold_test", "compressor_test", "comprex_test"])
+def test_cpp_mirror_of_reference_tests(name):
+    exe = os.path.join(BIN, name)
+    assert os.path.exists(exe), "build tests/cpp first (make -C tests/cpp, or __graft_entry__.build())"
+    print("running", exe, file=sys.stderr, flush=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    sys.stderr.write(r.stdout[-3000:] + r.stderr[-2000:])
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "+++ PASSED +++" in r.stdout and "--- FAILED ---" not in r.stdout
+
+
+def _pair(env, n, size_factor=3.0, topk=0.01, tag=1):
+    from comprex_amd import pygpi
+    objs = []
+    for rank in range(2):
+        env.set_rank(rank, 2)
+        c = pygpi.Comprex(env, n, size_factor)
+        c.setThreshold(pygpi.ThresholdTopK(topk))
+        c.setCompressor(pygpi.CompressorIndexPairs())
+        c.connectTo((rank + 1) % 2, (rank + 1) % 2, tag)
+        objs.append(c)
+    return objs
+
+
+@pytest.mark.parametrize("on_device", [False, True])
+def test_reference_abi_matches_oracle(oracle, on_device):
+    """Comprex.writeRemote / readRemote / flushRests through the reference's symbol set, against
+    the checker's writeRemote (default ThresholdTopK: 1000 strided samples), bit for bit."""
+    from comprex_amd import pygpi
+    n, topk = 200_003, np.float32(0.01)
+    env = pygpi.GaspiEnvironment()
+    tx, rx = _pair(env, n, topk=float(topk))
+    rng = np.random.default_rng(31)
+    rests = np.zeros(n, np.float32)
+    for it in range(6):
+        g = rng.standard_normal(n).astype(np.float32)
+        want_msg, want_thr = oracle.write_remote(rests, g, topk)
+        tx.writeRemote(torch.from_numpy(g).cuda() if on_device else g)
+        want_dense = np.zeros(n, np.float32)
+        oracle.ip_decompress(want_msg, want_dense)
+        if on_device:
+            got = torch.empty(n, device="cuda")
+            rx.readRemote(got)
+            got = got.cpu().numpy()
+        else:
+            got = rx.readRemote()
+        assert got.tobytes() == want_dense.tobytes()
+        assert tx.getRests().tobytes() == rests.tobytes()
+    want_flush = oracle.flush_rests(rests)
+    tx.flushRests()
+    acc = np.ones(n, np.float32)
+    want_acc = acc.copy()
+    oracle.ip_add(want_flush, want_acc)
+    rx.readRemote_add(acc)
+    assert acc.tobytes() == want_acc.tobytes()
+    assert not tx.getRests().any()
+
+
+def test_reference_abi_conservation_and_errors():
+    """test/comprex.cpp's gold through the Python wrappers, plus the errors the reference throws."""
+    from comprex_amd import pygpi
+    n = 50
+    env = pygpi.GaspiEnvironment()
+    tx, rx = _pair(env, n, topk=0.1)
+    i = np.arange(n)
+    values = (i * (1 - 2 * (i % 2))).astype(np.float32)
+    result = np.zeros(n, np.float32)
+    for run in range(4):
+        if run < 3:
+            tx.writeRemote(values)
+        else:
+            tx.flushRests()
+        rx.readRemote_add(result)
+    assert (result == 3 * values).all()
+    with pytest.raises(RuntimeError, match="no message pending"):
+        rx.readRemote()
+    with pytest.raises(RuntimeError):
+        tx.writeRemote(values[:-1].copy())
+    lone = pygpi.Comprex(env, n)
+    with pytest.raises(RuntimeError, match="without connecting"):
+        lone.writeRemote(values)
+    with pytest.raises(RuntimeError, match="between 0.0 and 1.0"):
+        pygpi.ThresholdTopK(1.5)
+    with pytest.raises(RuntimeError):
+        pygpi.ThresholdConst(-1.0)
+    t = pygpi.ThresholdConst(2.5)
+    assert t.getThreshold() == 2.5
+
+
+def test_simulated_all_to_one_reduce_matches_oracle(oracle):
+    """Config-5 shaped flow at a small size: R workers' messages reduced by the chief in rank
+    order (src/allreduce.tpp:183-189), then the chief's broadcast-leg writeRemote applies the
+    reduced vector to its residual (:205).  Checked against the checker's sequential loop."""
+    from comprex_amd import pygpi
+    R, n, topk = 5, 300_007, np.float32(0.01)
+    env = pygpi.GaspiEnvironment()
+    workers, chief_rx = [], []
+    for r in range(1, R):
+        env.set_rank(r, R)
+        w = pygpi.Comprex(env, n, 3.0)
+        w.setThreshold(pygpi.ThresholdTopK(float(topk)))
+        w.setCompressor(pygpi.CompressorIndexPairs())
+        w.connectTx(0, 100 + r)
+        workers.append(w)
+    env.set_rank(0, R)
+    for r in range(1, R):
+        c = pygpi.Comprex(env, n, 3.0)
+        c.setCompressor(pygpi.CompressorIndexPairs())
+        c.connectRx(r, 100 + r)
+        chief_rx.append(c)
+    bc = pygpi.Comprex(env, n, 3.0)
+    bc.setThreshold(pygpi.ThresholdTopK(float(topk)))
+    bc.setCompressor(pygpi.CompressorIndexPairs())
+    bc.connectTx(1, 200)
+    rng = np.random.default_rng(41)
+    o_rests = [np.zeros(n, np.float32) for _ in range(R)]
+    o_bc = np.zeros(n, np.float32)
+    for it in range(3):
+        grads = [rng.standard_normal(n).astype(np.float32) for _ in range(R)]
+        dense = torch.from_numpy(grads[0]).cuda()
+        want = grads[0].copy()
+        for r in range(1, R):
+            workers[r - 1].writeRemote(torch.from_numpy(grads[r]).cuda())
+            msg, _ = oracle.write_remote(o_rests[r], grads[r], topk)
+            oracle.ip_add(msg, want)
+        for r in range(1, R):
+            chief_rx[r - 1].readRemote_add(dense)
+        assert dense.cpu().numpy().tobytes() == want.tobytes()
+        bc.writeRemote(dense)
+        oracle.write_remote(o_bc, want, topk)
+        assert bc.getRests().tobytes() == o_bc.tobytes()
