@@ -22,6 +22,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 
 
+def measured_traffic(workload, n):
+    """Bytes per launch of the streaming kernel from the committed counter runs (FETCH_SIZE and
+    WRITE_SIZE, scaled by a plain copy of known size); None when they cover another workload."""
+    path = os.path.join(ROOT, "profiles", "stage_kernel_C4_100M_traffic.json")
+    try:
+        rec = json.load(open(path))
+    except (OSError, ValueError):
+        return None
+    return rec["traffic_bytes_per_launch"] if rec.get("workload") == workload and rec.get("n") == n else None
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -64,6 +75,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--items", type=int, default=None, help="compaction tile option (2/4/8)")
     ap.add_argument("--alternate", type=int, default=None, help="stage_alternate option (0/1)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device copy of the gradient (4n bytes read, 4n written) so that "
+                         "a counter run has a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU; the path has no inter-GPU part (--gpus %d refused)" % args.gpus)
@@ -102,6 +116,11 @@ def main():
     for _ in range(args.warmup):
         step()
     h.synchronize()
+    if args.calibrate_copy:
+        scratch = torch.empty_like(g)
+        scratch.copy_(g)
+        torch.cuda.synchronize()
+        del scratch
     # the library records a HIP event before and after its streaming kernel, on the stream it
     # launches on, for every step of the timed region
     h.set_option("profile_stage", 1)
@@ -198,7 +217,7 @@ def main():
         "config": {"workload": W.C4["name"], "n": n, "topK": float(topk), "sample_positions": m,
                    "threshold": "sampled ThresholdTopK over host-supplied positions", "input_checksum": W.checksum(g_h)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "stage_kernel<float,0,4,%d>"
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(W.C4["name"], n), "kernel": "stage_kernel<float,0,4,%d>"
                      % (args.items or 4), "algorithmic_bytes": kern_bytes, "avg_ms": kern_ms},
         "cpu_baseline": cpu,
         "extra": extra,

@@ -1,0 +1,163 @@
+"""The five benchmark configurations at their full sizes, on the GPU.
+
+Three kinds of evidence per configuration:
+  * the outputs of the COMPILED REFERENCE recorded in tests/golden/full_size.json (threshold
+    bits, pair count, checksums of message and residual), compared when the inputs regenerate
+    to the recorded checksum;
+  * the CPU checker run live on the same buffers where that takes seconds;
+  * size-independent properties (ascending indices, k == #{|r+g| > t}, conservation).
+"""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from comprex_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "full_size.json")))
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from comprex_amd.device import Handle
+    h = Handle()
+    yield h
+    h.synchronize()
+    h.close()
+
+
+def _msgbuf(n):
+    from comprex_amd.device import message_capacity
+    return torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+
+
+def _hex(x):
+    return np.float32(x).tobytes().hex()
+
+
+def _error_feedback(dev, oracle, cfg, grad_fn, iters, gold_rows, oracle_live=True):
+    n, topk, ds = cfg["n"], np.float32(cfg["topK"]), cfg["default_subsamples"]
+    rests = torch.zeros(n, device="cuda")
+    rests_h = np.zeros(n, np.float32)
+    buf = _msgbuf(n)
+    compared = 0
+    for it in range(iters):
+        g_h = grad_fn(it)
+        g = torch.from_numpy(g_h).cuda()
+        thr = dev.topk_threshold(rests, g, topk, ds)
+        nbytes = dev.compress(buf, g, rests)  # threshold from the handle's device slot
+        msg = buf[:nbytes].cpu().numpy()
+        k = int(msg[4:8].view(np.int32)[0])
+        say(cfg["name"], "iter", it, "thr", thr, "k", k)
+        idx = msg[8:].view(np.dtype([("i", np.int32), ("v", np.float32)]))["i"]
+        assert (np.diff(idx) > 0).all() and nbytes == 8 + 8 * k
+        if oracle_live:
+            want_msg, want_thr = oracle.write_remote(rests_h, g_h, topk, ds)
+            assert thr == want_thr and msg.tobytes() == want_msg.tobytes()
+            assert rests.cpu().numpy().tobytes() == rests_h.tobytes()
+        if it < len(gold_rows) and gold_rows[it]["input"] == W.checksum(g_h):
+            row = gold_rows[it]
+            assert _hex(thr) == row["thr_hex"] and k == row["k"]
+            assert W.checksum(msg) == row["msg"]
+            assert W.checksum(rests.cpu().numpy()) == row["rests"]
+            compared += 1
+    return compared
+
+
+def test_c1_one_million_top1pct_ten_iterations(dev, oracle):
+    compared = _error_feedback(dev, oracle, W.C1, W.c1_gradient, W.C1["iters"], GOLD["C1"])
+    assert compared == W.C1["iters"], "inputs did not regenerate to the recorded bits"
+
+
+def test_c2_lenet5_top10pct_fifty_iterations(dev, oracle):
+    compared = _error_feedback(dev, oracle, W.C2, W.c2_gradient, W.C2["iters"], GOLD["C2"])
+    assert compared == W.C2["iters"]
+
+
+def test_c3_resnet50_top0p1pct(dev, oracle):
+    # the first 3 of the 20 iterations carry recorded reference outputs and a live checker run
+    compared = _error_feedback(dev, oracle, W.C3, W.c3_gradient, 3, GOLD["C3"])
+    assert compared == 3
+
+
+def test_c4_hundred_million_laplace(dev, oracle):
+    g_h = W.c4_gradient()
+    n = g_h.size
+    assert W.checksum(g_h) == GOLD["C4"]["input"], "inputs did not regenerate to the recorded bits"
+    g = torch.from_numpy(g_h).cuda()
+    buf = _msgbuf(n)
+    topk = np.float32(W.C4["topK"])
+
+    def run(kind, thr_fn):
+        rests = torch.zeros(n, device="cuda")
+        thr = thr_fn(rests)
+        nbytes = dev.compress(buf, g, rests)
+        msg = buf[:nbytes].cpu().numpy()
+        k = int(msg[4:8].view(np.int32)[0])
+        row = GOLD["C4"][kind]
+        say("C4", kind, "thr", thr, "k", k)
+        assert _hex(thr) == row["thr_hex"] and k == row["k"]
+        assert W.checksum(msg) == row["msg"]
+        r = rests.cpu().numpy()
+        assert W.checksum(r) == row["rests"]
+        # properties: k == #{|g| > thr}; sent entries are +0 in the residual, the rest equals g
+        sel = np.abs(g_h) > np.float32(thr)
+        assert k == int(np.count_nonzero(sel))
+        idx = msg[8:].view(np.dtype([("i", np.int32), ("v", np.float32)]))["i"]
+        assert (idx == np.nonzero(sel)[0]).all()
+        assert not r[sel].any() and (r[~sel] == g_h[~sel]).all()
+        return rests
+
+    # reference-faithful strided sampling (1000 samples), exact top-k, and host-supplied positions
+    run("strided", lambda r: dev.topk_threshold(r, g, topk, 1000, 10.0))
+    run("exact", lambda r: dev.topk_threshold(r, g, topk, W.C4["default_subsamples_exact"], 10.0))
+    idx_h = W.c4_sample_indices()
+    assert W.checksum(idx_h) == GOLD["C4"]["indexed"]["idx"]
+    idx = torch.from_numpy(idx_h).cuda()
+    rests = run("indexed", lambda r: dev.topk_threshold_indexed(r, g, idx, topk))
+    # exact mode sends ceil_f32(n*topK)-1 pairs when no magnitude ties with the threshold
+    assert GOLD["C4"]["exact"]["k"] == 999_999
+
+    # conservation over error-feedback steps at full size: sum of decompressed messages + flush
+    # == steps * gradient, exact because every value here is a small multiple of 2^-10
+    q_h = np.round(g_h * 64).astype(np.float32) / np.float32(64)
+    q = torch.from_numpy(q_h).cuda()
+    rests.zero_()
+    total = torch.zeros(n, device="cuda")
+    for step in range(3):
+        dev.topk_threshold_indexed(rests, q, idx, topk, to_host=False)
+        dev.compress(buf, q, rests, sync=False)
+        dev.add(total, buf, check_header=False)
+    dev.compress(buf, rests, None, thr=0.0, sync=False)  # flushRests: data-only at threshold 0
+    dev.add(total, buf, check_header=False)
+    dev.synchronize()
+    assert torch.equal(total, q * 3)
+
+
+def test_c5_sparse_reduce_eight_ranks(dev, oracle):
+    msgs_h = W.c5_messages()
+    assert [W.checksum(m) for m in msgs_h] == GOLD["C5"]["msgs"], "inputs did not regenerate to the recorded bits"
+    n = W.C5["n"]
+    msgs = [torch.from_numpy(m).cuda() for m in msgs_h]
+    dense = torch.full((n,), 3.0, device="cuda")
+    dev.reduce(dense, msgs, accumulate=False, mode=0)
+    got = dense.cpu().numpy()
+    assert W.checksum(got) == GOLD["C5"]["dense"]  # rank-ordered: bit-exact with the reference
+    # atomics reorder the 8 contributions of the shared indices: 1e-6 relative (fp32)
+    dev.reduce(dense, msgs, accumulate=False, mode=1)
+    got_atomic = dense.cpu().numpy()
+    assert (np.abs(got_atomic - got) <= 1e-6 * 8 * np.maximum(np.abs(got), 1.0)).all()
+    # apply the reduced vector to a residual (addRests' loop) and compress it at 1 %
+    rests = torch.from_numpy(np.random.default_rng(9).standard_normal(n).astype(np.float32)).cuda()
+    want = rests.cpu().numpy() + got
+    dev.add_vec(rests, torch.from_numpy(got).cuda())
+    assert rests.cpu().numpy().tobytes() == want.tobytes()
+    dev.synchronize()
