@@ -200,6 +200,7 @@ int cx_destroy(cx_handle h) {
     if (h->tile_offsets) (void)hipFree(h->tile_offsets);
     if (h->block_sums) (void)hipFree(h->block_sums);
     if (h->redo_flag) (void)hipFree(h->redo_flag);
+    if (h->reduce_bounds) (void)hipFree(h->reduce_bounds);
     if (h->sel) (void)hipFree(h->sel);
     if (h->sel_keys) (void)hipFree(h->sel_keys);
     if (h->d_status) (void)hipFree(h->d_status);

@@ -80,6 +80,9 @@ struct cx_handle_s {
     unsigned epoch = 0;                // launch number
     unsigned parity = 0;               // flips every launch: which direction the pass walks
 
+    unsigned* reduce_bounds = nullptr;  // tiled reduce: first pair of each message in each dense tile
+    size_t reduce_bounds_cap = 0;
+
     cx::SelectState* sel = nullptr;
     void* sel_keys = nullptr;          // gathered sample keys of the two-launch select
     size_t sel_keys_bytes = 0;

@@ -309,6 +309,54 @@ def test_reduce_rank_order_bit_exact_and_atomic_tolerance(dev, oracle, dtype):
     dev.synchronize()
 
 
+def test_reduce_many_messages_duplicates_and_variants(dev, oracle):
+    """More messages than one tiled launch takes (16), repeated indices inside a message, empty
+    messages, a vector that ends inside a tile; both rank-ordered variants give the checker's bits."""
+    rng = np.random.default_rng(23)
+    n = 70_001
+    rec = np.dtype([("i", np.int32), ("v", np.float32)])
+    msgs = []
+    for r in range(20):
+        k = int(rng.integers(0, 900)) if r != 7 else 0
+        idx = np.sort(rng.integers(0, n, k)).astype(np.int32)  # sorted, repeats allowed
+        body = np.empty(k, rec)
+        body["i"], body["v"] = idx, rng.standard_normal(k).astype(np.float32) * np.float32(10.0 ** float(rng.integers(-3, 4)))
+        msgs.append(np.concatenate([np.array([n, k], np.int32).view(np.uint8), body.view(np.uint8)]))
+    base = rng.standard_normal(n).astype(np.float32)
+    gm = [_gpu(m) for m in msgs]
+    try:
+        for variant in (0, 1):
+            dev.set_option("reduce_variant", variant)
+            for accumulate in (False, True):
+                want = base.copy() if accumulate else np.zeros(n, np.float32)
+                for m in msgs:
+                    oracle.ip_add(m, want)
+                g = _gpu(base)
+                dev.reduce(g, gm, accumulate=accumulate, mode=0)
+                assert g.cpu().numpy().tobytes() == want.tobytes(), (variant, accumulate)
+            want = np.ones(n, np.float32)
+            oracle.ip_decompress(msgs[3], want)
+            g = torch.ones(n, device="cuda")
+            dev.decompress(g, gm[3])
+            assert g.cpu().numpy().tobytes() == want.tobytes()
+        dev.synchronize()
+    finally:
+        dev.set_option("reduce_variant", 0)
+
+
+def test_tiled_reduce_reports_unsorted_message(dev):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rec = np.dtype([("i", np.int32), ("v", np.float32)])
+    body = np.array([(5000, 1.0), (3, 2.0), (9000, 3.0)], dtype=rec)
+    msg = np.concatenate([np.array([10000, 3], np.int32).view(np.uint8), body.view(np.uint8)])
+    g = torch.zeros(10000, device="cuda")
+    dev.reduce(g, [_gpu(msg)], accumulate=False, mode=0)
+    with pytest.raises(ComprexError) as e:
+        dev.synchronize()
+    assert e.value.code == _lib.CX_ERR_INDEX
+
+
 # --------------------------------------------------------------------------- residual maintenance
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_zero_addvec_apply(dev, oracle, dtype):
