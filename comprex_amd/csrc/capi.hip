@@ -203,6 +203,7 @@ int cx_destroy(cx_handle h) {
     if (h->reduce_bounds) (void)hipFree(h->reduce_bounds);
     if (h->sel) (void)hipFree(h->sel);
     if (h->sel_keys) (void)hipFree(h->sel_keys);
+    if (h->cand) (void)hipFree(h->cand);
     if (h->d_status) (void)hipFree(h->d_status);
     if (h->d_thr) (void)hipFree(h->d_thr);
     if (h->h_pinned) (void)hipHostFree(h->h_pinned);
@@ -242,6 +243,8 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->profile_count = 0;
     } else if (!strcmp(key, "stage_alternate")) {
         h->stage_alternate = value ? 1 : 0;
+    } else if (!strcmp(key, "select_bracket")) {
+        h->select_bracket = value ? 1 : 0;
     } else if (!strcmp(key, "reduce_variant")) {
         h->reduce_variant = value;
     } else {

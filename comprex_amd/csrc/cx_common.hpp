@@ -78,12 +78,14 @@ struct cx_handle_s {
     size_t tiles_cap = 0;              // tiles allocated
     unsigned* redo_flag = nullptr;     // holds the launch number of the last launch that deferred a tile
     unsigned epoch = 0;                // launch number
-    unsigned parity = 0;               // flips every launch: which direction the pass walks
+    unsigned parity = 0;               // flips with every full pass over the vectors: 1 = the next one walks from the end
 
     unsigned* reduce_bounds = nullptr;  // tiled reduce: first pair of each message in each dense tile
     size_t reduce_bounds_cap = 0;
 
     cx::SelectState* sel = nullptr;
+    void* cand = nullptr;              // candidate keys of the one-pass whole-vector select
+    size_t cand_bytes = 0;
     void* sel_keys = nullptr;          // gathered sample keys of the two-launch select
     size_t sel_keys_bytes = 0;
     cx::DeviceStatus* d_status = nullptr;
@@ -99,6 +101,7 @@ struct cx_handle_s {
     // options
     int compact_items = 4;             // 16-byte loads per lane and tile
     int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
+    int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound
     int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
 };
 

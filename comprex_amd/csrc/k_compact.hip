@@ -430,6 +430,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     h->epoch += 1u;
     if (h->epoch == 0u) h->epoch = 1u;  // 0 is what a fresh flag holds
     unsigned* redo_flag = h->redo_flag;
+    const int reverse = h->stage_alternate ? (int)h->parity : 0;  // start where the previous full pass ended
     h->parity ^= 1u;
 
     const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
@@ -441,7 +442,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
                        (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, h->block_sums, redo_flag, h->epoch, ntiles,
-                       (h->stage_alternate && h->parity) ? 1 : 0);
+                       reverse);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
     // give the second pass the whole GPU instead of the gather kernel's few blocks

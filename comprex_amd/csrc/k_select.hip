@@ -15,6 +15,8 @@
 // compressor's `update[i] += data[i]` produces later).
 #include "cx_common.hpp"
 
+#include <cmath>
+
 namespace cx {
 
 namespace {
@@ -334,6 +336,102 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     }
 }
 
+// ---- whole-vector selection with a sampled lower bound ---------------------------------
+// Copies every key >= the key of *d_bound into `cand` (order irrelevant).  Each wavefront
+// gathers its matches in an LDS segment and appends the segment with ONE global atomic when it
+// fills up and at the end, so the counter sees a few thousand atomics per pass, not one per hit.
+// *cand_count keeps counting past `cap`; the host falls back when it overflows.
+constexpr int kCollectUnroll = 4;  // 16-byte loads in flight per lane
+
+template <typename T, bool HAS_ADD, int VEC>
+__global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                                long long m, const T* __restrict__ d_bound,
+                                                                typename Elem<T>::key_t* __restrict__ cand, unsigned cap,
+                                                                unsigned* __restrict__ cand_count, int reverse) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int kPerIter = 64 * VEC * kCollectUnroll;  // keys a wavefront looks at per iteration
+    constexpr int kSegKeys = 2 * kPerIter;
+    __shared__ key_t seg[kBlock / 64][kSegKeys];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const key_t bound = key_of(*d_bound);
+    key_t* my = seg[wave];
+    unsigned held = 0;  // keys in this wavefront's segment (same value in every lane)
+
+    auto flush = [&]() {
+        if (held == 0) return;
+        unsigned base = 0;
+        if (lane == 0) base = atomicAdd(cand_count, held);
+        base = __shfl(base, 0, 64);
+        for (unsigned i = lane; i < held; i += 64)
+            if (base + i < cap) cand[base + i] = my[i];
+        held = 0;
+    };
+    // appends this lane's hits (bit q of `mask` = key kk[q] is a candidate): one prefix sum over
+    // the lanes' hit counts places them; their order inside the segment does not matter
+    auto append = [&](const key_t* kk, unsigned mask, int nkeys) {
+        const unsigned cnt = __popc(mask);
+        unsigned incl = cnt;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const unsigned up = __shfl_up(incl, o, 64);
+            if (lane >= o) incl += up;
+        }
+        unsigned at = held + incl - cnt;
+        for (int q = 0; q < nkeys; ++q)
+            if ((mask >> q) & 1u) my[at++] = kk[q];
+        held += __shfl(incl, 63, 64);
+    };
+
+    const long long nvec = m / VEC;
+    const long long waves = (long long)gridDim.x * (kBlock / 64);
+    const long long wave_id = (long long)blockIdx.x * (kBlock / 64) + wave;
+    // a wavefront takes kCollectUnroll consecutive groups of 64 vectors per iteration; whole
+    // wavefronts stay in the loop together (cross-lane operations)
+    const long long ngroups = (nvec + 63) / 64;
+    for (long long g0 = wave_id * kCollectUnroll; g0 < ngroups; g0 += waves * kCollectUnroll) {
+        if (held + kPerIter > kSegKeys) flush();
+        Pack<T, VEC> a[kCollectUnroll], b[kCollectUnroll];
+        bool in[kCollectUnroll];
+#pragma unroll
+        for (int u = 0; u < kCollectUnroll; ++u) {
+            // reversed passes start at the far end, where the previous pass over the vectors ended
+            const long long g = reverse ? ngroups - 1 - (g0 + u) : g0 + u;
+            const long long i = g * 64 + lane;
+            in[u] = g >= 0 && i < nvec;
+            if (in[u]) {
+                a[u] = reinterpret_cast<const Pack<T, VEC>*>(vec)[i];
+                if (HAS_ADD) b[u] = reinterpret_cast<const Pack<T, VEC>*>(add)[i];
+            }
+        }
+        key_t kk[kCollectUnroll * VEC];
+        unsigned mask = 0;
+#pragma unroll
+        for (int u = 0; u < kCollectUnroll; ++u) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                T v = (T)0;
+                if (in[u]) v = HAS_ADD ? (T)(a[u].x[c] + b[u].x[c]) : a[u].x[c];
+                const key_t k = key_of(v);
+                kk[u * VEC + c] = k;
+                mask |= ((in[u] && k >= bound) ? 1u : 0u) << (u * VEC + c);
+            }
+        }
+        if (__any(mask != 0u)) append(kk, mask, kCollectUnroll * VEC);
+    }
+    if (blockIdx.x == 0 && wave == 0) {  // elements past the last full vector
+        const long long i = nvec * VEC + lane;
+        if (held + 64 > kSegKeys) flush();
+        T v = (T)0;
+        if (i < m) {
+            v = vec[i];
+            if (HAS_ADD) v = (T)(v + add[i]);
+        }
+        const key_t k = key_of(v);
+        append(&k, (i < m && k >= bound) ? 1u : 0u, 1);
+    }
+    flush();
+}
+
 template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v; }
 
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
@@ -363,21 +461,10 @@ void dispatch_hist(cx_handle h, int smode, bool vec_ok, const T* vec, const T* a
 
 }  // namespace
 
+// The key of descending rank `rank` among the m keys described by (vec, add_vec, d_idx, mode).
 template <typename T>
-int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
-                          float stepsize, float topK, T* d_thr_out) {
-    if (!d_thr_out) d_thr_out = static_cast<T*>(h->d_thr);
-    if (m <= 0) {
-        // empty input: undefined in the reference (dereferences end()); defined here as 1
-        hipLaunchKernelGGL(set_scalar_kernel<T>, dim3(1), dim3(1), 0, h->stream, d_thr_out, (T)1);
-        CX_HIP(hipGetLastError());
-        return CX_OK;
-    }
-    const int pos = cx_topk_pos((size_t)m, topK);
-    const int plus_one = pos <= 0 ? 1 : 0;
-    unsigned long long rank = plus_one ? 0ull : (unsigned long long)pos;
-    if (rank > (unsigned long long)(m - 1)) rank = (unsigned long long)(m - 1);
-
+int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
+                float stepsize, unsigned long long rank, int plus_one, T* d_thr_out) {
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
     using key_t = typename Elem<T>::key_t;
@@ -434,6 +521,87 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
     }
     CX_HIP(hipGetLastError());
     return CX_OK;
+}
+
+// Whole-vector selection in ONE pass over the vector(s) when the wanted rank is near the top:
+//   1. a strided sample gives a lower bound L that, with overwhelming probability, has at
+//      least rank+1 keys at or above it, and not many more;
+//   2. one pass copies the keys >= L into a candidate buffer;
+//   3. the host reads the candidate count (the only synchronisation); when rank < count <= capacity
+//      the answer is the key of the same rank among the candidates, found on that small set.
+// Otherwise *done stays 0 and the caller runs the full three-pass selection.  Exact either way.
+template <typename T>
+int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, unsigned long long rank, int plus_one,
+                          T* d_thr_out, int* done) {
+    using key_t = typename Elem<T>::key_t;
+    *done = 0;
+    constexpr int kSample = 1 << 16;
+    const double p = (double)(rank + 1) / (double)m;
+    const double expect = p * kSample;
+    const unsigned long long sample_rank = (unsigned long long)(expect + 8.0 * std::sqrt(expect) + 8.0);
+    const bool vec_ok = ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;
+    if (m < (1 << 23) || sample_rank >= (unsigned long long)kSample / 16 || !vec_ok) return CX_OK;
+
+    const size_t cap = (size_t)m / 16 > ((size_t)1 << 22) ? (size_t)m / 16 : ((size_t)1 << 22);
+    if (cap * sizeof(key_t) > h->cand_bytes) {
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->cand) CX_HIP(hipFree(h->cand));
+        h->cand = nullptr;
+        h->cand_bytes = 0;
+        CX_HIP(hipMalloc(&h->cand, cap * sizeof(key_t) + 256));
+        h->cand_bytes = cap * sizeof(key_t);
+    }
+    // 1. lower bound from the sample, left in the second half of the threshold slot
+    T* d_bound = reinterpret_cast<T*>(static_cast<char*>(h->d_thr) + 64);
+    unsigned* d_count = reinterpret_cast<unsigned*>(static_cast<char*>(h->d_thr) + 128);
+    const float stepsize = (float)m / (float)kSample;
+    int rc = select_rank<T>(h, vec, add_vec, m, nullptr, kSample, kSampleStrided, stepsize, sample_rank, 0, d_bound);
+    if (rc != CX_OK) return rc;
+    // 2. candidates; the pass starts at the end of the vectors where the previous pass stopped
+    const int reverse = h->stage_alternate ? (int)h->parity : 0;
+    h->parity ^= 1u;  // the next full pass (the compress that follows) walks the other way
+    CX_HIP(hipMemsetAsync(d_count, 0, sizeof(unsigned), h->stream));
+    constexpr int kVec = 16 / (int)sizeof(T);
+    key_t* cand = static_cast<key_t*>(h->cand);
+    if (add_vec)
+        hipLaunchKernelGGL((select_collect_kernel<T, true, kVec>), dim3(2048), dim3(kBlock), 0, h->stream, vec, add_vec,
+                           (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse);
+    else
+        hipLaunchKernelGGL((select_collect_kernel<T, false, kVec>), dim3(2048), dim3(kBlock), 0, h->stream, vec,
+                           add_vec, (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse);
+    CX_HIP(hipGetLastError());
+    // 3. how many?
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 12, d_count, sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
+    CX_HIP(hipStreamSynchronize(h->stream));
+    const unsigned long long count = (unsigned)h->h_pinned[12];
+    if (count <= rank || count > cap) return CX_OK;  // bound too high (or ties flooded the buffer): full selection
+    // magnitudes' bit patterns order like the magnitudes: the candidates are a vector of |x|
+    rc = select_rank<T>(h, reinterpret_cast<const T*>(cand), nullptr, (int)count, nullptr, (int)count, kSampleFull,
+                        1.0f, rank, plus_one, d_thr_out);
+    if (rc == CX_OK) *done = 1;
+    return rc;
+}
+
+template <typename T>
+int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
+                          float stepsize, float topK, T* d_thr_out) {
+    if (!d_thr_out) d_thr_out = static_cast<T*>(h->d_thr);
+    if (m <= 0) {
+        // empty input: undefined in the reference (dereferences end()); defined here as 1
+        hipLaunchKernelGGL(set_scalar_kernel<T>, dim3(1), dim3(1), 0, h->stream, d_thr_out, (T)1);
+        CX_HIP(hipGetLastError());
+        return CX_OK;
+    }
+    const int pos = cx_topk_pos((size_t)m, topK);
+    const int plus_one = pos <= 0 ? 1 : 0;
+    unsigned long long rank = plus_one ? 0ull : (unsigned long long)pos;
+    if (rank > (unsigned long long)(m - 1)) rank = (unsigned long long)(m - 1);
+    if (sample_mode == kSampleFull && h->select_bracket) {
+        int done = 0;
+        int rc = select_rank_bracketed<T>(h, vec, add_vec, m, rank, plus_one, d_thr_out, &done);
+        if (rc != CX_OK || done) return rc;
+    }
+    return select_rank<T>(h, vec, add_vec, n, d_idx, m, sample_mode, stepsize, rank, plus_one, d_thr_out);
 }
 
 template int launch_topk_threshold<float>(cx_handle, const float*, const float*, int, const int*, int, int, float, float, float*);

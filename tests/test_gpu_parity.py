@@ -184,6 +184,40 @@ def test_topk_threshold_matches_oracle(dev, oracle, dtype):
             assert dev.topk_threshold(gv, None, t, ds, sf) == want
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_exact_threshold_one_pass_bracket_and_fallbacks(dev, oracle, dtype):
+    """Whole-vector (exact top-k) thresholds on vectors large enough for the one-pass path
+    (sampled lower bound + candidate collection), including inputs that defeat the bound:
+    all-equal magnitudes (candidates overflow), a constant vector with a few outliers, and a
+    large topK (bracket not attempted).  Same bits as the checker, with the path on and off."""
+    rng = np.random.default_rng(19)
+    n = 9_000_001
+    ds = 1 << 24  # > n: exact mode
+    base = (rng.standard_normal(n) * 3).astype(dtype)
+    cases = {
+        "gauss": (base, 0.01),
+        "gauss_p0.001": (base, 0.001),
+        "gauss_p0.3": (base, 0.3),
+        "all_equal": (np.full(n, 2.5, dtype), 0.01),
+        "two_levels": (np.where(rng.random(n) < 0.004, 7.0, 1.0).astype(dtype), 0.01),
+        "ties_at_threshold": (np.round(base).astype(dtype), 0.02),
+    }
+    add = (rng.standard_normal(n) * 0.1).astype(dtype)
+    try:
+        for name, (v, topk) in cases.items():
+            t = np.float32(topk)
+            want_with = oracle.topk_prepare_with(v, add, t, ds, 10.0)
+            want = oracle.topk_prepare(v, t, ds, 10.0)
+            gv, ga = _gpu(v), _gpu(add)
+            for bracket in (1, 0):
+                say("exact threshold", dtype.__name__, name, "bracket", bracket)
+                dev.set_option("select_bracket", bracket)
+                assert dev.topk_threshold(gv, ga, t, ds, 10.0) == want_with
+                assert dev.topk_threshold(gv, None, t, ds, 10.0) == want
+    finally:
+        dev.set_option("select_bracket", 1)
+
+
 def test_topk_threshold_indexed_and_device_slot(dev, oracle):
     rng = np.random.default_rng(15)
     n, m = 1_000_000, 10_000
