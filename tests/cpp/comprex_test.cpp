@@ -123,6 +123,70 @@ template <typename data_t> int all_to_one(const char* name, int numRanks, int si
     return print_pass(errors);
 }
 
+// The send variants that leave the residual alone (src/comprEx.tpp:193-222) and the forwarders
+// of the ring schedules (:248-301), on a 3-rank chain 0 -> 1 -> 2 with the sizeBytes prefix on.
+template <typename data_t> int variants_and_forwarders(const char* name) {
+    const int size = 4000;
+    int errors = 0;
+    std::vector<data_t> values(size);
+    for (int i = 0; i < size; ++i) values[i] = (data_t)(((i * 37) % 201 - 100) * ((i % 3) ? 1 : 0));
+    GaspiEnvironment env(1 << 20);
+    std::vector<ComprEx<data_t> > c;
+    c.reserve(3);
+    for (int rank = 0; rank < 3; ++rank) {
+        env.set_rank(rank, 3);
+        c.emplace_back(env.get_segment(), size, 3.0f, true);
+        c[rank].setThreshold(ThresholdTopK<data_t>(0.05f, 1 << 13));  // exact top-k
+        c[rank].setCompressor(CompressorIndexPairs<data_t>());
+        c[rank].connectTo((rank + 2) % 3, (rank + 1) % 3, 5);  // receive from the left, send to the right
+    }
+    // writeRemote_compressOnly: every non-zero element arrives, residual stays zero
+    c[0].writeRemote_compressOnly(values.data(), size);
+    std::vector<data_t> got(size, (data_t)9);
+    c[1].readRemote(got.data(), size);
+    for (int i = 0; i < size; ++i) if (got[i] != values[i]) ++errors;
+    for (auto e : c[0].getRests()) if (e != 0) ++errors;
+    // writeRemote_NoResidual: threshold from the vector alone; |v| > thr arrives; residual untouched
+    ThresholdTopK<data_t> probe(0.05f, 1 << 13);
+    probe.prepare(values.data(), size);
+    const data_t thr = probe.get_threshold();
+    c[0].writeRemote_NoResidual(values.data(), size);
+    // rank 1 forwards the compressed message to rank 2 and decompresses it for itself
+    std::vector<data_t> at1(size, (data_t)9), at2(size, (data_t)9);
+    c[1].readRemote_forward(at1.data(), size);
+    c[2].readRemote(at2.data(), size);
+    int kept = 0;
+    for (int i = 0; i < size; ++i) {
+        const data_t want = std::abs(values[i]) > thr ? values[i] : (data_t)0;
+        if (want != 0) ++kept;
+        if (at1[i] != want || at2[i] != want) ++errors;
+    }
+    if (kept == 0 || kept > size / 10) ++errors;
+    for (auto e : c[0].getRests()) if (e != 0) ++errors;
+    // forward_buffer + forward_add (the big ring's hop, src/allreduce.tpp:663-675): rank 1 copies what it
+    // received into its own send buffer, sends it on and adds it to its vector
+    c[0].writeRemote(values.data(), size);  // residual += values, top 5 % sent
+    c[1].readRemote_wait();
+    c[1].forward_buffer();
+    std::vector<data_t> acc1(size, (data_t)1), acc2(size, (data_t)2);
+    c[1].forward_add(acc1.data(), size);
+    c[2].readRemote_add(acc2.data(), size);
+    std::vector<data_t> rests0 = c[0].getRests();
+    for (int i = 0; i < size; ++i) {
+        const data_t sent = values[i] - rests0[i];  // what left rank 0
+        if (acc1[i] != (data_t)1 + sent || acc2[i] != (data_t)2 + sent) ++errors;
+    }
+    // addRests / getRests(ptr) / resetRests
+    std::vector<data_t> plus(size, (data_t)3), copy(size);
+    c[0].addRests(plus.data(), size);
+    c[0].getRests(copy.data(), size);
+    for (int i = 0; i < size; ++i) if (plus[i] != (data_t)3 + rests0[i] || copy[i] != rests0[i]) ++errors;
+    c[0].resetRests();
+    for (auto e : c[0].getRests()) if (e != 0) ++errors;
+    std::cout << "send variants and forwarders (" << name << ")" << std::endl;
+    return print_pass(errors);
+}
+
 int error_paths() {
     int errors = 0;
     GaspiEnvironment env(1 << 20);
@@ -153,6 +217,8 @@ int main() {
     failed += comprex_p2p<double>("double");
     failed += all_to_one<int>("int", 4, 1000, 10, 0.01f);
     failed += all_to_one<float>("float", 3, 100000, 5, 0.001f);
+    failed += variants_and_forwarders<int>("int");
+    failed += variants_and_forwarders<float>("float");
     failed += error_paths();
     return failed ? 1 : 0;
 }
