@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <string>
 
+#include "../../include/allreduce.hxx"
 #include "../../include/comprEx.hxx"
 #include "../../include/compressor.hxx"
 #include "../../include/gaspiEnvironment.hxx"
@@ -59,6 +60,9 @@ void GaspiEnvironment_barrier(void* self) { static_cast<GaspiEnvironment*>(self)
 void GaspiEnvironment_flush(void* self) { static_cast<GaspiEnvironment*>(self)->flush(); }
 void GaspiEnvironment_set_rank(void* self, int rank, int ranks) {
     guarded([&] { static_cast<GaspiEnvironment*>(self)->set_rank(rank, ranks); });
+}
+void GaspiEnvironment_set_blocking(void* self, int blocking, double timeout_s) {
+    static_cast<GaspiEnvironment*>(self)->set_blocking(blocking != 0, timeout_s);
 }
 void Gaspi_Printf(const char* msg) {
     printf("%s\n", msg);
@@ -126,5 +130,45 @@ void* CompressorNone_new(void) { return new CompressorNone<data_t>(); }
 void CompressorNone_del(void* self) { delete static_cast<CompressorNone<data_t>*>(self); }
 void* CompressorIndexPairs_new(void) { return new CompressorIndexPairs<data_t>(); }
 void CompressorIndexPairs_del(void* self) { delete static_cast<CompressorIndexPairs<data_t>*>(self); }
+
+// ---- compressed allreduce schedules (src/allreduce_C.cpp:26-122) ----------------------------
+// One object per simulated rank, used from that rank's own thread (GaspiEnvironment_set_rank +
+// GaspiEnvironment_set_blocking); apply/flush work in place on `data` (host or device pointer).
+#define CX_ALLREDUCE_COMMON(NAME)                                                                        \
+    void* NAME##_new(void* gaspi_env) {                                                                  \
+        return guarded_value<void*>(nullptr, [&] { return (void*)new NAME<data_t>(static_cast<GaspiEnvironment*>(gaspi_env)); }); \
+    }                                                                                                    \
+    void NAME##_del(void* self) { delete static_cast<NAME<data_t>*>(self); }                             \
+    void NAME##_apply(void* self, float* data, int size) {                                               \
+        guarded([&] { static_cast<NAME<data_t>*>(self)->apply(data, size); });                           \
+    }                                                                                                    \
+    void NAME##_flush(void* self, float* data, int size) {                                               \
+        guarded([&] { static_cast<NAME<data_t>*>(self)->flush(data, size); });                           \
+    }                                                                                                    \
+    void NAME##_reset(void* self) { guarded([&] { static_cast<NAME<data_t>*>(self)->reset(); }); }       \
+    void NAME##_set_compression_ratio(void* self, float compression_ratio) {                             \
+        guarded([&] { static_cast<NAME<data_t>*>(self)->set_compression_ratio(compression_ratio); });    \
+    }
+CX_ALLREDUCE_COMMON(Comprex_AllToOneAllreduce)
+CX_ALLREDUCE_COMMON(Comprex_RingAllreduce)
+CX_ALLREDUCE_COMMON(Comprex_BigRingAllreduce)
+void Comprex_AllToOneAllreduce_setupConnections(void* self, int size, int tag, int chiefRank, float compression_ratio,
+                                                float size_factor) {
+    guarded([&] {
+        static_cast<Comprex_AllToOneAllreduce<data_t>*>(self)->setupConnections(size, tag, chiefRank, compression_ratio,
+                                                                                 size_factor);
+    });
+}
+void Comprex_RingAllreduce_setupConnections(void* self, int size, int tag, float compression_ratio, float size_factor) {
+    guarded([&] {
+        static_cast<Comprex_RingAllreduce<data_t>*>(self)->setupConnections(size, tag, compression_ratio, size_factor);
+    });
+}
+void Comprex_BigRingAllreduce_setupConnections(void* self, int size, int tag, float compression_ratio,
+                                               float size_factor) {
+    guarded([&] {
+        static_cast<Comprex_BigRingAllreduce<data_t>*>(self)->setupConnections(size, tag, compression_ratio, size_factor);
+    });
+}
 
 }  // extern "C"

@@ -32,9 +32,18 @@ _PROTOS = {
     "ThresholdConst_getThreshold": (_f, [_vp]),
     "ThresholdTopK_new": (_vp, [_f]), "ThresholdTopK_del": (None, [_vp]),
     "ThresholdTopK_getThreshold": (_f, [_vp]),
+    "GaspiEnvironment_set_blocking": (None, [_vp, _i, C.c_double]),
     "CompressorNone_new": (_vp, []), "CompressorNone_del": (None, [_vp]),
     "CompressorIndexPairs_new": (_vp, []), "CompressorIndexPairs_del": (None, [_vp]),
 }
+for _fam, _setup in (("Comprex_AllToOneAllreduce", [_vp, _i, _i, _i, _f, _f]),
+                     ("Comprex_RingAllreduce", [_vp, _i, _i, _f, _f]),
+                     ("Comprex_BigRingAllreduce", [_vp, _i, _i, _f, _f])):
+    _PROTOS.update({
+        _fam + "_new": (_vp, [_vp]), _fam + "_del": (None, [_vp]), _fam + "_setupConnections": (None, _setup),
+        _fam + "_apply": (None, [_vp, _vp, _i]), _fam + "_flush": (None, [_vp, _vp, _i]),
+        _fam + "_reset": (None, [_vp]), _fam + "_set_compression_ratio": (None, [_vp, _f]),
+    })
 _bound = None
 
 
@@ -89,6 +98,10 @@ class GaspiEnvironment(Getable):
         """Not in the reference: which simulated rank the following calls act as."""
         libcomprex().GaspiEnvironment_set_rank(self.obj, rank, ranks)
         _raise_if_failed()
+
+    def set_blocking(self, blocking, timeout_s=60.0):
+        """Not in the reference: one host thread per rank; receives wait for their message."""
+        libcomprex().GaspiEnvironment_set_blocking(self.obj, int(blocking), float(timeout_s))
 
     def barrier(self):
         libcomprex().GaspiEnvironment_barrier(self.obj)
@@ -216,3 +229,73 @@ class CompressorIndexPairs(Getable):
 
     def __del__(self):
         libcomprex().CompressorIndexPairs_del(self.obj)
+
+
+###########################
+# Compressed allreduce schedules (allreduce.py:175-355 of the reference)
+###########################
+class _ComprexAllreduce(Getable):
+    _family = None
+
+    def __init__(self, gaspi_env):
+        self.env = gaspi_env
+        self.size = None
+        self.obj = getattr(libcomprex(), self._family + "_new")(gaspi_env.get())
+        _raise_if_failed()
+
+    def __del__(self):
+        if getattr(self, "obj", None):
+            getattr(libcomprex(), self._family + "_del")(self.obj)
+            self.obj = None
+
+    def apply(self, vector):
+        """In place on `vector` (float32 numpy array or CUDA tensor); returns it."""
+        p, n = _ptr_size(vector)
+        getattr(libcomprex(), self._family + "_apply")(self.obj, p, n)
+        _raise_if_failed()
+        return vector
+
+    def flush(self, vector):
+        p, n = _ptr_size(vector)
+        getattr(libcomprex(), self._family + "_flush")(self.obj, p, n)
+        _raise_if_failed()
+        return vector
+
+    def reset(self):
+        getattr(libcomprex(), self._family + "_reset")(self.obj)
+        _raise_if_failed()
+
+    def set_compression_ratio(self, compression_ratio):
+        getattr(libcomprex(), self._family + "_set_compression_ratio")(self.obj, compression_ratio)
+        _raise_if_failed()
+
+    def getSize(self):
+        return self.size
+
+
+class Comprex_AllToOneAllreduce(_ComprexAllreduce):
+    _family = "Comprex_AllToOneAllreduce"
+
+    def setup_connections(self, size, tag, chiefRank, compression_ratio, size_factor=1.0):
+        self.size = size
+        libcomprex().Comprex_AllToOneAllreduce_setupConnections(self.obj, size, tag, chiefRank, compression_ratio,
+                                                               size_factor)
+        _raise_if_failed()
+
+
+class Comprex_RingAllreduce(_ComprexAllreduce):
+    _family = "Comprex_RingAllreduce"
+
+    def setup_connections(self, size, tag, compression_ratio, size_factor=1.0):
+        self.size = size
+        libcomprex().Comprex_RingAllreduce_setupConnections(self.obj, size, tag, compression_ratio, size_factor)
+        _raise_if_failed()
+
+
+class Comprex_BigRingAllreduce(_ComprexAllreduce):
+    _family = "Comprex_BigRingAllreduce"
+
+    def setup_connections(self, size, tag, compression_ratio, size_factor=1.0):
+        self.size = size
+        libcomprex().Comprex_BigRingAllreduce_setupConnections(self.obj, size, tag, compression_ratio, size_factor)
+        _raise_if_failed()

@@ -9,7 +9,8 @@
 //     (source, target, tag) triple, owned by the GaspiEnvironment stand-in: the sender's
 //     compressor writes the message where the receiver reads it, ordered by the HIP stream;
 //   * `vector` arguments may be host pointers (staged) or device pointers (used in place);
-//   * a receive with no message pending throws instead of blocking for ever;
+//   * with one thread playing all ranks a receive with no message pending throws instead of
+//     blocking for ever; with one thread per rank (GaspiEnvironment::set_blocking) it waits;
 //   * writeRemote only enqueues GPU work; nothing is copied to the host.
 #ifndef COMPREX_H
 #define COMPREX_H
@@ -47,6 +48,7 @@ protected:
 
     cxx::Handle handle_;
     cxx::DeviceBuffer stage_;
+    cxx::DeviceBuffer forward_;  // message in transit between inbox and outbox (forward_buffer)
 
     VarTYPE* rests() const { return static_cast<VarTYPE*>(restsVect.data()); }
     char* src_address() const { return static_cast<char*>(srcBuff_data->buffer.data()); }
@@ -60,9 +62,11 @@ protected:
 
     // "waitForCompletion" of the reference's TargetBuffer
     void wait_for_message() {
-        if (targBuff_data->received >= targBuff_data->sent)
-            throw std::runtime_error("Receive issued with no message pending (the reference would block here)!");
-        targBuff_data->received = targBuff_data->sent;
+        targBuff_data->wait_message(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s());
+    }
+    // the source buffer may be overwritten once the receiver has read the previous message
+    void wait_for_room() {
+        srcBuff_data->wait_consumed(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s());
     }
 
     // send-side tail shared by all write paths: data-only / update-only / fused compression
@@ -130,8 +134,9 @@ public:
     // Sends the whole residual (no thresholding: every non-zero element) and clears it.
     virtual void flushRests() {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        wait_for_room();
         compress_into(0, rests(), nullptr, rests_size, false);
-        srcBuff_data->sent += 1;
+        srcBuff_data->post();
         resetRests();
     }
 
@@ -193,8 +198,9 @@ public:
                      rests_size, size);
             throw std::runtime_error(msg);
         }
+        wait_for_room();
         compress_into(0, v.get(), rests(), rests_size, true);
-        srcBuff_data->sent += 1;
+        srcBuff_data->post();
     }
 
     // compression only: no threshold, residual untouched
@@ -202,8 +208,9 @@ public:
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
+        wait_for_room();
         compress_into(0, v.get(), nullptr, size, false);
-        srcBuff_data->sent += 1;
+        srcBuff_data->post();
     }
 
     // threshold from the vector alone, residual untouched
@@ -212,8 +219,9 @@ public:
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
         threshold->prepare(v.get(), size);
+        wait_for_room();
         compress_into(0, v.get(), nullptr, size, true);
-        srcBuff_data->sent += 1;
+        srcBuff_data->post();
     }
 
     // overwrites `vector` with the received message
@@ -222,6 +230,7 @@ public:
         wait_for_message();
         const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
         compressor->decompress(vector, size, targ_address() + offset);
+        targBuff_data->consumed();
     }
 
     // adds the received message to `vector`
@@ -230,62 +239,75 @@ public:
         wait_for_message();
         const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
         compressor->add(vector, size, targ_address() + offset);
+        targBuff_data->consumed();
     }
 
     // receive, pass the compressed message on to this object's target, and decompress it
     void readRemote_forward(VarTYPE* vector, int size) {
         wait_for_message();
+        wait_for_room();
         cx_handle h = handle_.get();
         if (send_sizeBytes) {
             int sizeBytes = 0;
             cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
             cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
-            srcBuff_data->sent += 1;
+            srcBuff_data->post();
             compressor->decompress(vector, size, targ_address() + sizeof(int));
         } else {
             const int sizeBytes = compressor->decompress(vector, size, targ_address());
             cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes));
-            srcBuff_data->sent += 1;
+            srcBuff_data->post();
         }
+        targBuff_data->consumed();
     }
 
     void readRemote_forwardCopy(VarTYPE* vector, int size) {
         if (!this->send_sizeBytes)
             throw std::runtime_error("If using readRemote_forwardCopy, send_sizeBytes must be true!");
         wait_for_message();
+        wait_for_room();
         cx_handle h = handle_.get();
         int sizeBytes = 0;
         cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
         cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
+        targBuff_data->consumed();
     }
 
     void readRemote_wait() { wait_for_message(); }
 
+    // copies the received message into the send buffer (it is sent by forward_add).  The copy
+    // goes through a private buffer: the inbox is released before this object waits for room in
+    // its outbox, so a ring of ranks that all forward at once cannot wait on each other in a circle
+    // (the reference has separate source and target buffers and feedback tokens for this).
     void forward_buffer() {
         if (!this->send_sizeBytes) throw std::runtime_error("If using forward_buffer, send_sizeBytes must be true!");
         cx_handle h = handle_.get();
         int sizeBytes = 0;
         cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
-        cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
+        const size_t bytes = (size_t)sizeBytes + sizeof(int);
+        void* hold = forward_.reserve(bytes);
+        cxx::check(cx_copy(h, hold, targ_address(), bytes));
+        targBuff_data->consumed();
+        wait_for_room();
+        cxx::check(cx_copy(h, src_address(), hold, bytes));
     }
 
+    // sends the message sitting in the send buffer and adds it to `vector`
     void forward_add(VarTYPE* vector, int size) {
         if (!this->send_sizeBytes) throw std::runtime_error("If using forward_add, send_sizeBytes must be true!");
-        srcBuff_data->sent += 1;
         compressor->add(vector, size, src_address() + sizeof(int));
+        srcBuff_data->post();
     }
 
     virtual void connectTx(int targRank, int tag) {
         this->targRank = targRank;
         alloc_rests();  // the residual exists only on objects that send
         srcBuff_data = gaspiCxx_segment->channel(gaspiCxx_segment->get_rank(), targRank, tag, bufferSize);
-        srcBuff_data->has_sender = true;
     }
 
     virtual void connectRx(int srcRank, int tag) {
         this->srcRank = srcRank;
         targBuff_data = gaspiCxx_segment->channel(srcRank, gaspiCxx_segment->get_rank(), tag, bufferSize);
-        targBuff_data->has_receiver = true;
     }
 
     // srcRank: receive data from this rank; targRank: send data to this rank
@@ -312,6 +334,11 @@ protected:
     using ComprEx<VarTYPE>::restsVect;
     using ComprEx<VarTYPE>::srcBuff_data;
 
+public:
+    using ComprEx<VarTYPE>::writeRemote_compressOnly;  // the const overload stays visible
+
+protected:
+
     long long send_offset() const { return doublebuffer_offset * ((doublebuffer_phase + 1) % 2); }
     long long write_offset() const { return doublebuffer_offset * doublebuffer_phase; }
     void update_doublebuffer_phase() { doublebuffer_phase = (doublebuffer_phase + 1) % 2; }
@@ -324,12 +351,13 @@ protected:
     // "initTransferPart(sizeBytes, send_offset)": hand the half at `off` to the receiver
     void send_half(long long off) {
         cx_handle h = this->handle_.get();
+        this->wait_for_room();
         // the message's own header tells its length; copy header first, then the pairs it announces
         int hdr[2] = {0, 0};
         cxx::check(cx_copy(h, hdr, half(off), 8));
         const size_t bytes = 8 + (size_t)(hdr[1] < 0 ? 0 : hdr[1]) * (4 + sizeof(VarTYPE));
         cxx::check(cx_copy(h, this->src_address(), half(off), bytes));
-        srcBuff_data->sent += 1;
+        srcBuff_data->post();
     }
 
     void compress_half(long long off, const VarTYPE* d_data, VarTYPE* d_update, int n, bool use_threshold) {

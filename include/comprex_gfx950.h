@@ -203,6 +203,34 @@ void* CompressorNone_new(void);
 void CompressorNone_del(void* self);
 void* CompressorIndexPairs_new(void);
 void CompressorIndexPairs_del(void* self);
+/* src/allreduce_C.cpp:26-122, the three compressed schedules.  One object per simulated rank, driven
+ * from that rank's own host thread (GaspiEnvironment_set_rank, then GaspiEnvironment_set_blocking so
+ * that receives wait for their message); apply/flush work in place on `data`, host or device. */
+void GaspiEnvironment_set_blocking(void* self, int blocking, double timeout_s);
+void* Comprex_AllToOneAllreduce_new(void* gaspi_env);
+void Comprex_AllToOneAllreduce_del(void* self);
+void Comprex_AllToOneAllreduce_setupConnections(void* self, int size, int tag, int chiefRank, float compression_ratio,
+                                                float size_factor);
+void Comprex_AllToOneAllreduce_apply(void* self, float* data, int size);
+void Comprex_AllToOneAllreduce_flush(void* self, float* data, int size);
+void Comprex_AllToOneAllreduce_reset(void* self);
+void Comprex_AllToOneAllreduce_set_compression_ratio(void* self, float compression_ratio);
+void* Comprex_RingAllreduce_new(void* gaspi_env);
+void Comprex_RingAllreduce_del(void* self);
+void Comprex_RingAllreduce_setupConnections(void* self, int size, int tag, float compression_ratio, float size_factor);
+void Comprex_RingAllreduce_apply(void* self, float* data, int size);
+void Comprex_RingAllreduce_flush(void* self, float* data, int size);
+void Comprex_RingAllreduce_reset(void* self);
+void Comprex_RingAllreduce_set_compression_ratio(void* self, float compression_ratio);
+void* Comprex_BigRingAllreduce_new(void* gaspi_env);
+void Comprex_BigRingAllreduce_del(void* self);
+void Comprex_BigRingAllreduce_setupConnections(void* self, int size, int tag, float compression_ratio,
+                                               float size_factor);
+void Comprex_BigRingAllreduce_apply(void* self, float* data, int size);
+void Comprex_BigRingAllreduce_flush(void* self, float* data, int size);
+void Comprex_BigRingAllreduce_reset(void* self);
+void Comprex_BigRingAllreduce_set_compression_ratio(void* self, float compression_ratio);
+
 /* Error text of the last reference-ABI call that failed on this thread ("" if none).  The
  * reference lets std::runtime_error escape through extern "C"; here it is caught. */
 const char* Comprex_lastError(void);

@@ -15,7 +15,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "cpp", "bin")
 
 
-@pytest.mark.parametrize("name", ["threshold_test", "compressor_test", "comprex_test"])
+@pytest.mark.parametrize("name", ["threshold_test", "compressor_test", "comprex_test", "allreduce_test"])
 def test_cpp_mirror_of_reference_tests(name):
     exe = os.path.join(BIN, name)
     assert os.path.exists(exe), "build tests/cpp first (make -C tests/cpp, or __graft_entry__.build())"
@@ -146,3 +146,56 @@ def test_simulated_all_to_one_reduce_matches_oracle(oracle):
         bc.writeRemote(dense)
         oracle.write_remote(o_bc, want, topk)
         assert bc.getRests().tobytes() == o_bc.tobytes()
+
+
+@pytest.mark.parametrize("family", ["Comprex_AllToOneAllreduce", "Comprex_RingAllreduce", "Comprex_BigRingAllreduce"])
+def test_allreduce_schedules_from_python_threads(family):
+    """The reference's Python allreduce tests (test/AllToOneAllreduce.py etc.): one thread per rank,
+    device tensors handed to apply/flush in place, gold (num_runs*(numRanks-1)+1)*values."""
+    import threading
+    from comprex_amd import pygpi
+    R, n, runs = 3, 30_000, 4
+    env = pygpi.GaspiEnvironment()
+    env.set_rank(0, R)
+    env.set_blocking(True, 60.0)
+    i = np.arange(n)
+    values = ((i % 251) * (1 - 2 * (i % 2))).astype(np.float32)
+    gold = (runs * (R - 1) + 1) * values
+    results, errors = {}, []
+
+    def rank_program(rank):
+        try:
+            env.set_rank(rank, R)
+            ar = getattr(pygpi, family)(env)
+            if family == "Comprex_AllToOneAllreduce":
+                ar.setup_connections(n, 0, 0, 1e-2, 3.0)
+            else:
+                ar.setup_connections(n, 0, 1e-2, 3.0)
+            env.barrier()
+            result = torch.from_numpy(values).cuda()
+            for run in range(runs):
+                env.barrier()
+                if family == "Comprex_RingAllreduce":
+                    seg = n // R
+                    lo = ((rank + 1) % R) * seg
+                    keep = result[lo:lo + seg].clone()
+                    result.copy_(torch.from_numpy(values))
+                    result[lo:lo + seg] = keep
+                elif rank != 0:
+                    result.copy_(torch.from_numpy(values))
+                ar.apply(result)
+            ar.flush(result)
+            results[rank] = result.cpu().numpy()
+            env.barrier()
+        except Exception as e:  # noqa: BLE001
+            errors.append((rank, repr(e)))
+
+    threads = [threading.Thread(target=rank_program, args=(r,)) for r in range(R)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(120)
+    assert not errors, errors
+    checked = range(R) if family == "Comprex_RingAllreduce" else [0]
+    for r in checked:
+        assert (results[r] == gold).all(), (family, r)
