@@ -167,6 +167,23 @@ def main():
         extra["exact_topk_GBps"] = (20 * n + 8 * kx + 8) / (ex_ms * 1e-3) / 1e9
         extra["exact_topk_k"] = kx
         log("exact top-k step %.3f ms (%.0f GB/s of 20n+8k+8), k=%d" % (ex_ms, extra["exact_topk_GBps"], kx))
+        # the same as one call: exact threshold and compress in a single pass over the vectors
+        rests.zero_()
+        for _ in range(2):
+            h.compress_topk(msg, g, rests, topk)
+        t0 = time.perf_counter()
+        routes = []
+        for _ in range(reps):
+            h.compress_topk(msg, g, rests, topk)  # waits for the stream itself
+            routes.append(h.get_option("fused_topk_taken"))
+        fx_ms = (time.perf_counter() - t0) / reps * 1e3
+        kf = int(hdr[1].item())
+        extra["exact_topk_fused_step_ms"] = fx_ms
+        extra["exact_topk_fused_GBps"] = (20 * n + 8 * kf + 8) / (fx_ms * 1e-3) / 1e9
+        extra["exact_topk_fused_k"] = kf
+        extra["exact_topk_fused_routes"] = sorted(set(routes))
+        log("exact top-k, single pass: %.3f ms (%.0f GB/s of 20n+8k+8), k=%d, routes %s"
+            % (fx_ms, extra["exact_topk_fused_GBps"], kf, extra["exact_topk_fused_routes"]))
         del g, rests, msg
         torch.cuda.empty_cache()
 

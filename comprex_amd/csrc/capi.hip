@@ -107,6 +107,18 @@ int compress_impl(cx_handle h, void* out_msg, long long out_capacity, const void
 }
 
 template <typename T>
+int compress_topk_impl(cx_handle h, void* out_msg, long long out_capacity, const void* data, void* update, int n,
+                       float topK, void* d_thr_out, int* d_size_prefix, int* h_bytes) {
+    int rc = launch_compress_topk<T>(h, out_msg, out_capacity, static_cast<const T*>(data), static_cast<T*>(update), n,
+                                     topK, static_cast<T*>(d_thr_out), d_size_prefix);
+    if (rc != CX_OK || !h_bytes) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, out_msg, 8, hipMemcpyDeviceToHost, h->stream));
+    rc = collect_status(h);
+    *h_bytes = 8 + h->h_pinned[9] * 4 * Elem<T>::pair_words;
+    return rc;
+}
+
+template <typename T>
 int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_bytes) {
     int rc = launch_decompress<T>(h, static_cast<T*>(out), out_n, msg);
     if (rc != CX_OK || !h_bytes) return rc;
@@ -247,9 +259,24 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->select_bracket = value ? 1 : 0;
     } else if (!strcmp(key, "reduce_variant")) {
         h->reduce_variant = value;
+    } else if (!strcmp(key, "fused_topk")) {
+        h->fused_topk = value ? 1 : 0;
     } else {
         return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     }
+    return CX_OK;
+}
+
+int cx_get_option(cx_handle h, const char* key, int* value) {
+    if (!h || !key || !value) return fail(CX_ERR_INVALID, "null handle, key or output");
+    if (!strcmp(key, "compact_items")) *value = h->compact_items;
+    else if (!strcmp(key, "profile_stage")) *value = h->profile;
+    else if (!strcmp(key, "stage_alternate")) *value = h->stage_alternate;
+    else if (!strcmp(key, "select_bracket")) *value = h->select_bracket;
+    else if (!strcmp(key, "reduce_variant")) *value = h->reduce_variant;
+    else if (!strcmp(key, "fused_topk")) *value = h->fused_topk;
+    else if (!strcmp(key, "fused_topk_taken")) *value = h->fused_topk_taken;
+    else return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     return CX_OK;
 }
 
@@ -312,6 +339,15 @@ int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capaci
                    int n, const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
     if (!h) return fail(CX_ERR_INVALID, "null handle");
     CX_DISPATCH(dt, compress_impl<T>(h, out_msg, out_capacity, data, update, n, thr_host, d_thr, d_size_prefix, h_bytes));
+}
+
+int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
+                        int n, float topK, void* d_thr_out, int* d_size_prefix, int* h_bytes) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (n < 0 || !update || !data) return fail(CX_ERR_INVALID, "compress_topk: needs both vectors and a size >= 0");
+    if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
+    CX_DISPATCH(dt, compress_topk_impl<T>(h, out_msg, out_capacity, data, update, n, topK, d_thr_out, d_size_prefix,
+                                          h_bytes));
 }
 
 int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes) {

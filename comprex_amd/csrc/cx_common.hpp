@@ -84,7 +84,7 @@ struct cx_handle_s {
     size_t reduce_bounds_cap = 0;
 
     cx::SelectState* sel = nullptr;
-    void* cand = nullptr;              // candidate keys of the one-pass whole-vector select
+    void* cand = nullptr;              // candidates of the one-pass whole-vector select (keys) / fused top-k (pairs)
     size_t cand_bytes = 0;
     void* sel_keys = nullptr;          // gathered sample keys of the two-launch select
     size_t sel_keys_bytes = 0;
@@ -102,6 +102,8 @@ struct cx_handle_s {
     int compact_items = 4;             // 16-byte loads per lane and tile
     int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
     int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound
+    int fused_topk = 1;                // 1 = cx_ip_compress_topk may take its single-pass route
+    int fused_topk_taken = 0;          // how the last cx_ip_compress_topk ran: 0 two calls, 1 single pass, 2 single pass abandoned
     int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
 };
 
@@ -115,6 +117,17 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
 template <typename T>
 int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m,
                           int sample_mode, float stepsize, float topK, T* d_thr_out);
+
+// fused exact top-k (whole-vector ThresholdTopK + compress_add_update in one pass over the vectors)
+template <typename T>
+int launch_candidates(cx_handle h, unsigned* cand_words, long long cap_pairs, const T* data, T* update, int n,
+                      const T* d_bound);
+template <typename T>
+int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, const T* d_thr,
+                  T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result);
+template <typename T>
+int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
+                         float topK, T* d_thr_out, int* d_size_prefix);
 
 template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg);
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);

@@ -100,7 +100,9 @@ __device__ __forceinline__ void put_pair(unsigned* w, unsigned index, double v) 
 
 // One wavefront, one tile.  MODE 0: update += data, select on update, zero selected
 // (compress_add_update); MODE 1: select on update, zero selected (compress_update);
-// MODE 2: select on data, nothing written back (compress).
+// MODE 2: select on data, nothing written back (compress); MODE 3: update += data, select on
+// update, nothing zeroed (candidate pass of the fused exact top-k: the selected set is a superset
+// of what is finally sent, and the residual must survive a change of plan untouched).
 // DIRECT false: stage the pairs (or defer the tile); true: write them at `direct_pos`.
 template <typename T, int MODE, int VEC, int ITEMS, bool DIRECT>
 __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* __restrict__ update, long long n,
@@ -128,7 +130,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         unsigned valid = (1u << VEC) - 1u;
         if (full) {
             if (MODE != 2) u = load_pack<T, VEC>(update + e0, false);
-            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
+            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);  // MODE 3 reads both
         } else {
             valid = 0;
 #pragma unroll
@@ -144,7 +146,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
             T v;
-            if (MODE == 0) v = (T)(u.x[c] + d.x[c]);
+            if (MODE == 0 || MODE == 3) v = (T)(u.x[c] + d.x[c]);
             else if (MODE == 1) v = u.x[c];
             else v = d.x[c];
             s[j][c] = v;
@@ -195,15 +197,16 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
                 else overflow = true;
                 ++pos;
             }
-            w.x[c] = keep ? (T)0 : s[j][c];
+            w.x[c] = (keep && MODE != 3) ? (T)0 : s[j][c];
         }
         if (MODE != 2) {
             if (full) {
-                if (MODE == 0 || m != 0u) store_pack<T, VEC>(update + e0, w, CX_NT_UPDATE_STORE != 0);
+                if (MODE == 0 || MODE == 3 || m != 0u) store_pack<T, VEC>(update + e0, w, CX_NT_UPDATE_STORE != 0);
             } else {
 #pragma unroll
                 for (int c = 0; c < VEC; ++c)
-                    if (((valid_mask[j] >> c) & 1u) && (MODE == 0 || ((m >> c) & 1u))) update[e0 + c] = w.x[c];
+                    if (((valid_mask[j] >> c) & 1u) && (MODE == 0 || MODE == 3 || ((m >> c) & 1u)))
+                        update[e0 + c] = w.x[c];
             }
         }
     }
@@ -420,7 +423,7 @@ int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
 
 template <typename T, int MODE, int VEC, int ITEMS>
 int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
-               long long cap_pairs, int* size_prefix) {
+               long long cap_pairs, int* size_prefix, DeviceStatus* status) {
     constexpr int kTile = 64 * VEC * ITEMS;
     constexpr int kCap = kTile / 8;
     constexpr int PW = Elem<T>::pair_words;
@@ -451,12 +454,12 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
                        update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->block_sums,
                        h->tile_offsets, h->staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
-                       h->d_status);
+                       status);
     if (dense_hint) {
         const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
         hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
                            update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->tile_offsets, redo_flag, h->epoch,
-                           ntiles, msg_words + 2, cap_pairs, h->d_status);
+                           ntiles, msg_words + 2, cap_pairs, status);
     }
     CX_HIP(hipGetLastError());
     return CX_OK;
@@ -465,9 +468,13 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
 template <typename T, int VEC, int ITEMS>
 int launch_mode(cx_handle h, int mode, const T* data, T* update, int n, const T* thr_ptr, T thr_val,
                 unsigned* msg_words, long long cap_pairs, int* size_prefix) {
-    if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
-    if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
-    return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix);
+    DeviceStatus* st = h->d_status;
+    if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
+    if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
+    if (mode == 2) return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
+    // candidate pass: an overflowing candidate buffer is a change of plan, not an error of the caller
+    return launch_all<T, 3, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix,
+                                        reinterpret_cast<DeviceStatus*>(static_cast<char*>(h->d_thr) + 192));
 }
 
 }  // namespace
@@ -503,6 +510,173 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
         default: return fail(CX_ERR_INVALID, "compress: unsupported compact_items %d", h->compact_items);
     }
 }
+
+// ---- fused exact top-k: candidate pass and final filter -------------------------------------
+// Candidate pass: update += data (nothing zeroed) and every element with |update| > *d_bound as an
+// (index, value) pair, ascending, behind a message header in `cand_words`.
+template <typename T>
+int launch_candidates(cx_handle h, unsigned* cand_words, long long cap_pairs, const T* data, T* update, int n,
+                      const T* d_bound) {
+    constexpr int kVec = 16 / (int)sizeof(T);
+    switch (h->compact_items) {
+        case 2: return launch_mode<T, kVec, 2>(h, 3, data, update, n, d_bound, (T)0, cand_words, cap_pairs, nullptr);
+        case 4: return launch_mode<T, kVec, 4>(h, 3, data, update, n, d_bound, (T)0, cand_words, cap_pairs, nullptr);
+        case 8: return launch_mode<T, kVec, 8>(h, 3, data, update, n, d_bound, (T)0, cand_words, cap_pairs, nullptr);
+        default: return fail(CX_ERR_INVALID, "compress: unsupported compact_items %d", h->compact_items);
+    }
+}
+
+namespace {
+
+constexpr int kFilterBlocks = 2048;
+constexpr int kFilterBlock = 256;
+
+template <typename T> __device__ __forceinline__ T pair_value(const unsigned* w);
+template <> __device__ __forceinline__ float pair_value<float>(const unsigned* w) { return __uint_as_float(w[1]); }
+template <> __device__ __forceinline__ int pair_value<int>(const unsigned* w) { return (int)w[1]; }
+template <> __device__ __forceinline__ double pair_value<double>(const unsigned* w) {
+    return __longlong_as_double((long long)((unsigned long long)w[1] | ((unsigned long long)w[2] << 32)));
+}
+
+// The candidate list is usable when it holds the wanted order statistic (more candidates than
+// the rank) and nothing was dropped from it.
+__device__ __forceinline__ bool candidates_usable(unsigned count, unsigned cap, unsigned long long rank) {
+    return (unsigned long long)count > rank && count <= cap;
+}
+
+// Survivors (|value| > threshold) per block-sized share of the candidate list.
+template <typename T>
+__global__ __launch_bounds__(kFilterBlock) void filter_count_kernel(const unsigned* __restrict__ cand_words,
+                                                                    unsigned cand_cap, unsigned long long rank,
+                                                                    const T* __restrict__ thr_ptr,
+                                                                    unsigned* __restrict__ block_counts) {
+    constexpr int PW = Elem<T>::pair_words;
+    __shared__ unsigned s_cnt;
+    if (threadIdx.x == 0) s_cnt = 0u;
+    __syncthreads();
+    const unsigned count = cand_words[1];
+    unsigned mine = 0;
+    if (candidates_usable(count, cand_cap, rank)) {
+        const unsigned share = (count + kFilterBlocks - 1) / kFilterBlocks;
+        const unsigned lo = blockIdx.x * share;
+        const unsigned hi = lo + share < count ? lo + share : count;
+        const T thr = *thr_ptr;
+        for (unsigned i = lo + threadIdx.x; i < hi; i += kFilterBlock)
+            mine += mag(pair_value<T>(cand_words + 2 + (size_t)i * PW)) > thr ? 1u : 0u;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mine += __shfl_xor(mine, off, 64);
+    if ((threadIdx.x & 63) == 0) atomicAdd(&s_cnt, mine);  // LDS
+    __syncthreads();
+    if (threadIdx.x == 0) block_counts[blockIdx.x] = s_cnt;
+}
+
+// Copies the survivors to the message in list order and clears their residual entries; the last
+// block writes the header.  result[0]: 0 = done, 1 = candidate list not usable (nothing written);
+// result[1]: pairs in the message, or the candidate count.
+template <typename T>
+__global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
+    const unsigned* __restrict__ cand_words, unsigned cand_cap, unsigned long long rank, const T* __restrict__ thr_ptr,
+    const unsigned* __restrict__ block_counts, T* __restrict__ update, int n, unsigned* __restrict__ msg_words,
+    long long cap_pairs, int* __restrict__ size_prefix, unsigned* __restrict__ result, DeviceStatus* status) {
+    constexpr int PW = Elem<T>::pair_words;
+    constexpr int kWaves = kFilterBlock / 64;
+    __shared__ unsigned s_before;
+    __shared__ unsigned s_wave[kWaves];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const unsigned count = cand_words[1];
+    if (!candidates_usable(count, cand_cap, rank)) {
+        if (blockIdx.x == 0 && tid == 0) {
+            result[0] = 1u;
+            result[1] = count;
+        }
+        return;
+    }
+    if (tid == 0) s_before = 0u;
+    __syncthreads();
+    unsigned before = 0;
+    for (unsigned b = tid; b < blockIdx.x; b += kFilterBlock) before += block_counts[b];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
+    if (lane == 0 && before) atomicAdd(&s_before, before);  // LDS
+    __syncthreads();
+    unsigned pos = s_before;  // survivors before the part of the share not yet walked
+
+    const unsigned share = (count + kFilterBlocks - 1) / kFilterBlocks;
+    const unsigned lo = blockIdx.x * share;
+    const unsigned hi = lo + share < count ? lo + share : count;
+    const T thr = *thr_ptr;
+    const unsigned long long below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    unsigned* const pairs = msg_words + 2;
+    bool overflow = false;
+    for (unsigned i0 = lo; i0 < hi; i0 += kFilterBlock) {  // uniform trip count per block
+        const unsigned i = i0 + tid;
+        unsigned w[PW];
+        bool keep = false;
+        if (i < hi) {
+#pragma unroll
+            for (int q = 0; q < PW; ++q) w[q] = cand_words[2 + (size_t)i * PW + q];
+            keep = mag(pair_value<T>(w)) > thr;
+        }
+        const unsigned long long votes = __ballot(keep);
+        if (lane == 0) s_wave[wave] = (unsigned)__popcll(votes);
+        __syncthreads();
+        unsigned at = pos + (unsigned)__popcll(votes & below);
+        unsigned all = 0;
+#pragma unroll
+        for (int q = 0; q < kWaves; ++q) {
+            if (q < wave) at += s_wave[q];
+            all += s_wave[q];
+        }
+        if (keep) {
+            if ((long long)at < cap_pairs) {
+#pragma unroll
+                for (int q = 0; q < PW; ++q) pairs[(size_t)at * PW + q] = w[q];
+            } else {
+                overflow = true;
+            }
+            if (w[0] < (unsigned)n) update[w[0]] = (T)0;
+        }
+        pos += all;
+        __syncthreads();
+    }
+    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    if (blockIdx.x == kFilterBlocks - 1 && tid == 0) {
+        msg_words[0] = (unsigned)n;
+        msg_words[1] = pos;
+        if (size_prefix) *size_prefix = (int)(8u + pos * (unsigned)(4 * PW));
+        result[0] = 0u;
+        result[1] = pos;
+    }
+}
+
+}  // namespace
+
+// Final step of the fused exact top-k: the candidates above *d_thr become the message and leave
+// the residual; nothing happens (result[0] = 1) when the candidate list cannot hold the answer.
+template <typename T>
+int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, const T* d_thr,
+                  T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result) {
+    // per-share counts live behind the per-block sums of the streaming pass, which are consumed by now
+    int rc = ensure_scratch(h, (size_t)kFilterBlocks * kWavesPerBlock, 0);
+    if (rc != CX_OK) return rc;
+    hipLaunchKernelGGL(filter_count_kernel<T>, dim3(kFilterBlocks), dim3(kFilterBlock), 0, h->stream, cand_words,
+                       cand_cap, rank, d_thr, h->block_sums);
+    hipLaunchKernelGGL(filter_write_kernel<T>, dim3(kFilterBlocks), dim3(kFilterBlock), 0, h->stream, cand_words,
+                       cand_cap, rank, d_thr, h->block_sums, update, n, msg_words, cap_pairs, size_prefix, d_result,
+                       h->d_status);
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
+#define CX_INSTANTIATE_FUSED(T)                                                                                      \
+    template int launch_candidates<T>(cx_handle, unsigned*, long long, const T*, T*, int, const T*);                 \
+    template int launch_filter<T>(cx_handle, const unsigned*, unsigned, unsigned long long, const T*, T*, int,       \
+                                  unsigned*, long long, int*, unsigned*);
+CX_INSTANTIATE_FUSED(float)
+CX_INSTANTIATE_FUSED(double)
+CX_INSTANTIATE_FUSED(int)
+#undef CX_INSTANTIATE_FUSED
 
 template int launch_compact<float>(cx_handle, void*, long long, const float*, float*, int, const float*, const float*, int*);
 template int launch_compact<double>(cx_handle, void*, long long, const double*, double*, int, const double*, const double*, int*);

@@ -36,193 +36,29 @@ __device__ __forceinline__ float value_of(uint32_t k, float) { return __uint_as_
 __device__ __forceinline__ double value_of(uint64_t k, double) { return __longlong_as_double((long long)k); }
 __device__ __forceinline__ int value_of(uint32_t k, int) { return (int)k; }
 
-__global__ __launch_bounds__(kBlock) void select_init_kernel(SelectState* st, unsigned long long rank) {
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) st->hist[b] = 0u;
-    if (threadIdx.x == 0) {
-        st->prefix = 0ull;
-        st->mask = 0ull;
-        st->rank = rank;
-    }
-}
-
-// One histogram pass.  SMODE: 0 whole vector, 1 strided, 2 indexed.
-template <typename T, int SMODE, bool HAS_ADD, int VEC>
-__global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
-                                                             const int* __restrict__ idx, long long m, int n,
-                                                             float stepsize, SelectState* __restrict__ st, int shift,
-                                                             int bits) {
-    using key_t = typename Elem<T>::key_t;
-    __shared__ unsigned lds_hist[kRadixBins];
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
-    __syncthreads();
-
-    const key_t prefix = (key_t)st->prefix;
-    const key_t mask = (key_t)st->mask;
-    const unsigned digit_mask = (1u << bits) - 1u;
-    const long long stride = (long long)gridDim.x * kBlock;
-
-    if (SMODE == 0 && VEC > 1) {
-        const long long nvec = m / VEC;
-        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) {
-            Pack<T, VEC> a = reinterpret_cast<const Pack<T, VEC>*>(vec)[i];
-            if (HAS_ADD) {
-                Pack<T, VEC> b = reinterpret_cast<const Pack<T, VEC>*>(add)[i];
-#pragma unroll
-                for (int c = 0; c < VEC; ++c) a.x[c] = (T)(a.x[c] + b.x[c]);
-            }
-#pragma unroll
-            for (int c = 0; c < VEC; ++c) {
-                const key_t k = key_of(a.x[c]);
-                if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
-            }
-        }
-        // tail elements
-        for (long long i = nvec * VEC + (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
-            T v = vec[i];
-            if (HAS_ADD) v = (T)(v + add[i]);
-            const key_t k = key_of(v);
-            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
-        }
-    } else {
-        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
-            long long p;
-            bool ok = true;
-            if (SMODE == 0) {
-                p = i;
-            } else if (SMODE == 1) {
-                // (int)(i * stepsize), product rounded to fp32 (threshold.hxx:217,236)
-                p = (long long)(int)__fmul_rn((float)(int)i, stepsize);
-                if (p > (long long)n - 1) p = (long long)n - 1;  // the reference would read out of bounds
-                if (p < 0) p = 0;
-            } else {
-                p = idx[i];
-                ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
-                if (!ok) p = 0;
-            }
-            T v = vec[p];
-            if (HAS_ADD) v = (T)(v + add[p]);
-            const key_t k = ok ? key_of(v) : (key_t)0;
-            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
-        }
-    }
-    __syncthreads();
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
-        const unsigned c = lds_hist[b];
-        if (c) atomicAdd(&st->hist[b], c);
-    }
-}
-
-// Picks the digit that holds the wanted descending rank, narrows the state, clears the
-// histogram for the next pass.  After the last pass the key is complete and the
-// threshold is written.  One block.
-template <typename T>
-__global__ __launch_bounds__(kBlock) void select_pick_kernel(SelectState* st, int shift, int bits, int last,
-                                                             int plus_one, T* __restrict__ thr_out) {
-    constexpr int kPer = kRadixBins / kBlock;  // bins per thread
-    __shared__ unsigned long long s_sum[kBlock];
-    __shared__ unsigned s_digit;
-    __shared__ unsigned long long s_above;
-    const int t = threadIdx.x;
-    // thread t owns bins [hi - kPer + 1, hi], walking from the top digit down
-    const int hi = kRadixBins - 1 - t * kPer;
-    unsigned cnt[kPer];
-    unsigned long long local = 0;
-#pragma unroll
-    for (int q = 0; q < kPer; ++q) {
-        cnt[q] = st->hist[hi - q];
-        local += cnt[q];
-    }
-    s_sum[t] = local;
-    if (t == 0) {
-        s_digit = 0u;
-        s_above = 0ull;
-    }
-    __syncthreads();
-    // exclusive scan over threads (256 values; serial per thread is cheap enough: one block, once per pass)
-    unsigned long long before = 0;
-    for (int q = 0; q < t; ++q) before += s_sum[q];
-    const unsigned long long rank = st->rank;
-    if (rank >= before && rank < before + local) {
-        unsigned long long acc = before;
-#pragma unroll
-        for (int q = 0; q < kPer; ++q) {
-            if (rank < acc + cnt[q]) {
-                s_digit = (unsigned)(hi - q);
-                s_above = acc;
-                break;
-            }
-            acc += cnt[q];
-        }
-    }
-    __syncthreads();
-    for (int b = t; b < kRadixBins; b += kBlock) st->hist[b] = 0u;
-    if (t == 0) {
-        const unsigned long long digit_mask = ((1ull << bits) - 1ull) << shift;
-        const unsigned long long prefix = st->prefix | ((unsigned long long)s_digit << shift);
-        st->prefix = prefix;
-        st->mask = st->mask | digit_mask;
-        st->rank = rank - s_above;
-        if (last) {
-            using key_t = typename Elem<T>::key_t;
-            T v = value_of((key_t)prefix, T());
-            if (plus_one) v = (T)(v + 1);
-            *thr_out = v;
-        }
-    }
-}
-
-// ---- small sample sets: two launches ---------------------------------------------------
-// First launch: one thread per sample gathers its key, stores it to `keys` and counts the
-// top digit (LDS histogram merged into the global one).  Second launch, one block: picks the
-// top digit, then finishes the remaining digits over the stored keys with LDS histograms only.
-constexpr int kFinishBlock = 1024;
-
-template <typename T, int SMODE, bool HAS_ADD>
-__global__ __launch_bounds__(kBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
-                                                              const int* __restrict__ idx, int m, int n, float stepsize,
-                                                              typename Elem<T>::key_t* __restrict__ keys,
-                                                              SelectState* __restrict__ st, int shift, int bits) {
-    using key_t = typename Elem<T>::key_t;
-    __shared__ unsigned lds_hist[kRadixBins];
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
-    __syncthreads();
-    const unsigned digit_mask = (1u << bits) - 1u;
-    const int stride = gridDim.x * kBlock;
-    for (int i = blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
-        long long p;
-        bool ok = true;
-        if (SMODE == 0) {
-            p = i;
-        } else if (SMODE == 1) {
-            p = (long long)(int)__fmul_rn((float)i, stepsize);  // (int)(i * stepsize), product in fp32
-            if (p > (long long)n - 1) p = (long long)n - 1;     // the reference would read out of bounds
-            if (p < 0) p = 0;
-        } else {
-            p = idx[i];
-            ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
-            if (!ok) p = 0;
-        }
-        T v = vec[p];
-        if (HAS_ADD) v = (T)(v + add[p]);
-        const key_t k = ok ? key_of(v) : (key_t)0;
-        keys[i] = k;
-        atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
-    }
-    __syncthreads();
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
-        const unsigned c = lds_hist[b];
-        if (c) atomicAdd(&st->hist[b], c);
-    }
+// ---- pieces shared by the selection kernels ------------------------------------------------
+// Digit count into an LDS histogram.  The keys a wavefront looks at together often share one
+// digit (candidates just above a bound, samples of one exponent): those are counted with ONE
+// atomic.  Must be called by whole wavefronts.
+__device__ __forceinline__ void hist_add(unsigned* lds_hist, bool active, unsigned digit) {
+    const unsigned long long act = __ballot(active);
+    if (act == 0ull) return;
+    const int leader = __ffsll((long long)act) - 1;
+    const unsigned d0 = __shfl(digit, leader, 64);
+    const unsigned long long same = __ballot(active && digit == d0);
+    if ((int)(threadIdx.x & 63) == leader) atomicAdd(&lds_hist[d0], (unsigned)__popcll(same));
+    if (active && digit != d0) atomicAdd(&lds_hist[digit], 1u);
 }
 
 // Block-wide: digit holding descending rank `rank` in hist[0..kRadixBins), and how many keys
-// lie above that digit.  All threads get the result.
+// lie above that digit.  All threads get the result.  A rank beyond the total gives digit 0.
+template <int BLOCK>
 __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long long rank, unsigned long long* s_sum,
                                            unsigned* s_digit, unsigned long long* s_above, unsigned& digit,
                                            unsigned long long& above) {
-    constexpr int kPer = kRadixBins / kFinishBlock;  // 2 bins per thread
+    constexpr int kPer = kRadixBins / BLOCK;  // bins per thread
     const int t = threadIdx.x;
-    const int hi = kRadixBins - 1 - t * kPer;
+    const int hi = kRadixBins - 1 - t * kPer;  // thread t owns bins [hi - kPer + 1, hi], top digits first
     unsigned cnt[kPer];
     unsigned long long local = 0;
 #pragma unroll
@@ -230,8 +66,7 @@ __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long l
         cnt[q] = hist[hi - q];
         local += cnt[q];
     }
-    // inclusive scan over threads, top digits first
-    unsigned long long incl = local;
+    unsigned long long incl = local;  // inclusive scan over threads
     const int lane = t & 63, wave = t >> 6;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -264,6 +99,211 @@ __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long l
     __syncthreads();
 }
 
+__global__ __launch_bounds__(kBlock) void select_init_kernel(SelectState* st, unsigned long long rank) {
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) st->hist[b] = 0u;
+    if (threadIdx.x == 0) {
+        st->prefix = 0ull;
+        st->mask = 0ull;
+        st->rank = rank;
+    }
+}
+
+// Adds a block's LDS digit counts to the global histogram.
+template <int BLOCK> __device__ __forceinline__ void merge_hist(const unsigned* lds_hist, SelectState* st) {
+    __syncthreads();
+    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) {
+        const unsigned c = lds_hist[b];
+        if (c) atomicAdd(&st->hist[b], c);
+    }
+}
+
+// Picks the digit that holds the wanted descending rank, narrows the state, clears the
+// histogram for the next pass.  After the last pass the key is complete and the
+// threshold is written.  One block.  (Folding this into the histogram kernel, with the block
+// that arrives last doing the pick, was measured slower on this GPU: the device-scope fences
+// that make the other blocks' counts visible inside one kernel cost more than a launch.)
+template <typename T>
+__global__ __launch_bounds__(kBlock) void select_pick_kernel(SelectState* st, int shift, int bits, int last,
+                                                             int plus_one, T* __restrict__ thr_out) {
+    __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit;
+    __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+        lds_hist[b] = st->hist[b];
+        st->hist[b] = 0u;
+    }
+    __syncthreads();
+    const unsigned long long rank = st->rank;
+    unsigned digit;
+    unsigned long long above;
+    block_pick<kBlock>(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+    if (threadIdx.x == 0) {
+        const unsigned long long prefix = st->prefix | ((unsigned long long)digit << shift);
+        st->prefix = prefix;
+        st->mask = st->mask | (((1ull << bits) - 1ull) << shift);
+        st->rank = rank - above;
+        if (last) {
+            using key_t = typename Elem<T>::key_t;
+            T v = value_of((key_t)prefix, T());
+            if (plus_one) v = (T)(v + 1);
+            *thr_out = v;
+        }
+    }
+}
+
+// One histogram pass over the keys described by (vec, add, idx).  SMODE: 0 whole vector,
+// 1 strided, 2 indexed.
+template <typename T, int SMODE, bool HAS_ADD, int VEC>
+__global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                             const int* __restrict__ idx, long long m, int n,
+                                                             float stepsize, SelectState* __restrict__ st, int shift,
+                                                             int bits) {
+    using key_t = typename Elem<T>::key_t;
+    __shared__ unsigned lds_hist[kRadixBins];
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    __syncthreads();
+
+    const key_t prefix = (key_t)st->prefix;
+    const key_t mask = (key_t)st->mask;
+    const unsigned digit_mask = (1u << bits) - 1u;
+    const long long stride = (long long)gridDim.x * kBlock;
+
+    if (SMODE == 0 && VEC > 1) {
+        const long long nvec = m / VEC;
+        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) {
+            Pack<T, VEC> x = reinterpret_cast<const Pack<T, VEC>*>(vec)[i];
+            if (HAS_ADD) {
+                Pack<T, VEC> y = reinterpret_cast<const Pack<T, VEC>*>(add)[i];
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) x.x[c] = (T)(x.x[c] + y.x[c]);
+            }
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) {
+                const key_t k = key_of(x.x[c]);
+                if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+            }
+        }
+        // tail elements
+        for (long long i = nvec * VEC + (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
+            T v = vec[i];
+            if (HAS_ADD) v = (T)(v + add[i]);
+            const key_t k = key_of(v);
+            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+        }
+    } else {
+        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
+            long long p;
+            bool ok = true;
+            if (SMODE == 0) {
+                p = i;
+            } else if (SMODE == 1) {
+                // (int)(i * stepsize), product rounded to fp32 (threshold.hxx:217,236)
+                p = (long long)(int)__fmul_rn((float)(int)i, stepsize);
+                if (p > (long long)n - 1) p = (long long)n - 1;  // the reference would read out of bounds
+                if (p < 0) p = 0;
+            } else {
+                p = idx[i];
+                ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+                if (!ok) p = 0;
+            }
+            T v = vec[p];
+            if (HAS_ADD) v = (T)(v + add[p]);
+            const key_t k = ok ? key_of(v) : (key_t)0;
+            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+        }
+    }
+    merge_hist<kBlock>(lds_hist, st);
+}
+
+// One histogram pass over the values of an IndexPairs message (int32 n | int32 k | k pairs), whose
+// pair count is only known on the device; at most `cap` pairs are looked at.
+template <typename T> __device__ __forceinline__ typename Elem<T>::key_t pair_key(const unsigned* w);
+template <> __device__ __forceinline__ uint32_t pair_key<float>(const unsigned* w) { return w[1] & 0x7fffffffu; }
+template <> __device__ __forceinline__ uint32_t pair_key<int>(const unsigned* w) { return key_of((int)w[1]); }
+template <> __device__ __forceinline__ uint64_t pair_key<double>(const unsigned* w) {
+    return ((uint64_t)w[1] | ((uint64_t)w[2] << 32)) & 0x7fffffffffffffffull;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigned* __restrict__ msg_words, unsigned cap,
+                                                                   SelectState* __restrict__ st, int shift, int bits) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int PW = Elem<T>::pair_words;
+    __shared__ unsigned lds_hist[kRadixBins];
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    __syncthreads();
+    const key_t prefix = (key_t)st->prefix;
+    const key_t mask = (key_t)st->mask;
+    const unsigned digit_mask = (1u << bits) - 1u;
+    unsigned m = msg_words[1];
+    if (m > cap) m = cap;
+    const unsigned stride = gridDim.x * kBlock;
+    // whole wavefronts stay in the loop together (hist_add is a cross-lane operation); four
+    // independent loads per lane are in flight before the first count
+    for (unsigned i0 = blockIdx.x * kBlock; i0 < m; i0 += 4u * stride) {
+        key_t k[4];
+        bool in[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const unsigned i = i0 + (unsigned)q * stride + threadIdx.x;
+            in[q] = i < m;  // m <= cap < 2^31 / 4: the index cannot wrap
+            k[q] = in[q] ? pair_key<T>(msg_words + 2 + (size_t)i * PW) : (key_t)0;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            hist_add(lds_hist, in[q] && (k[q] & mask) == prefix, (unsigned)(k[q] >> shift) & digit_mask);
+    }
+    merge_hist<kBlock>(lds_hist, st);
+}
+
+// ---- small sample sets: two launches ---------------------------------------------------
+// First launch: one thread per sample gathers its key, stores it to `keys` and counts the top
+// digit.  Second launch, one block: picks the top digit and finishes the remaining digits alone;
+// when the keys sharing the picked top digit fit in LDS they are collected there in one scan of
+// `keys` and the other passes never leave LDS, else every pass scans `keys` again.
+constexpr int kFinishBlock = 1024;
+
+template <typename T, int SMODE, bool HAS_ADD>
+__global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                              const int* __restrict__ idx, int m, int n, float stepsize,
+                                                              typename Elem<T>::key_t* __restrict__ keys,
+                                                              SelectState* __restrict__ st) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
+    __shared__ unsigned lds_hist[kRadixBins];
+    // large blocks: every block ends with one global atomic per digit it has seen, and those
+    // queue up per address
+    for (int b = threadIdx.x; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
+    __syncthreads();
+    const int stride = gridDim.x * kFinishBlock;
+    // whole wavefronts stay in the loop together (hist_add is a cross-lane operation)
+    for (int i0 = blockIdx.x * kFinishBlock; i0 < m; i0 += stride) {
+        const int i = i0 + threadIdx.x;
+        key_t k = 0;
+        if (i < m) {
+            long long p;
+            bool ok = true;
+            if (SMODE == 0) {
+                p = i;
+            } else if (SMODE == 1) {
+                p = (long long)(int)__fmul_rn((float)i, stepsize);  // (int)(i * stepsize), product in fp32
+                if (p > (long long)n - 1) p = (long long)n - 1;     // the reference would read out of bounds
+                if (p < 0) p = 0;
+            } else {
+                p = idx[i];
+                ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+                if (!ok) p = 0;
+            }
+            T v = vec[p];
+            if (HAS_ADD) v = (T)(v + add[p]);
+            k = ok ? key_of(v) : (key_t)0;
+            keys[i] = k;
+        }
+        hist_add(lds_hist, i < m, (unsigned)(k >> shift0) & ((1u << kRadixBits) - 1u));
+    }
+    merge_hist<kFinishBlock>(lds_hist, st);
+}
+
 template <typename T>
 __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typename Elem<T>::key_t* __restrict__ keys,
                                                                      int m, SelectState* __restrict__ st,
@@ -272,10 +312,11 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
+    constexpr int kListKeys = 32768 / (int)sizeof(key_t);
     __shared__ unsigned lds_hist[kRadixBins];
-    __shared__ unsigned long long s_sum[kFinishBlock / 64];
-    __shared__ unsigned s_digit;
-    __shared__ unsigned long long s_above;
+    __shared__ key_t s_list[kListKeys];
+    __shared__ unsigned s_digit, s_fill;
+    __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
     const int t = threadIdx.x;
 
     // top digit: counted by the first launch into the global histogram
@@ -285,6 +326,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     }
     __syncthreads();
     key_t prefix = 0, mask = 0;
+    unsigned listed = 0;  // keys in s_list (0 = scan `keys`)
     for (int p = 0; p < kPasses; ++p) {
         int shift = kKeyBits - kRadixBits * (p + 1);
         int bits = kRadixBits;
@@ -292,42 +334,75 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             bits += shift;
             shift = 0;
         }
+        const unsigned digit_mask = (1u << bits) - 1u;
         if (p > 0) {
             for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
             __syncthreads();
-            const unsigned digit_mask = (1u << bits) - 1u;
-            constexpr int KV = 16 / (int)sizeof(key_t);  // keys per 16-byte load
-            const int nvec = m / KV;
-            const Pack<key_t, KV>* kv = reinterpret_cast<const Pack<key_t, KV>*>(keys);
-            for (int v0 = 0; v0 < nvec; v0 += kFinishBlock * 4) {
-                Pack<key_t, KV> kk[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int v = v0 + q * kFinishBlock + t;
-                    if (v < nvec) kk[q] = kv[v];
+            if (listed) {
+                for (unsigned i = t; i < listed; i += kFinishBlock) {
+                    const key_t k1 = s_list[i];
+                    if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 }
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (v0 + q * kFinishBlock + t < nvec) {
-#pragma unroll
-                        for (int c = 0; c < KV; ++c)
-                            if ((kk[q].x[c] & mask) == prefix)
-                                atomicAdd(&lds_hist[(unsigned)(kk[q].x[c] >> shift) & digit_mask], 1u);
-                    }
+            } else {
+                for (int i = t; i < m; i += kFinishBlock) {
+                    const key_t k1 = keys[i];
+                    if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 }
-            }
-            for (int i = nvec * KV + t; i < m; i += kFinishBlock) {
-                const key_t k1 = keys[i];
-                if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
             }
             __syncthreads();
         }
         unsigned digit;
         unsigned long long above;
-        block_pick(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+        block_pick<kFinishBlock>(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+        const unsigned in_digit = lds_hist[digit];
         prefix |= (key_t)digit << shift;
         mask |= (key_t)((1ull << bits) - 1ull) << shift;
         rank -= above;
+        if (p == 0 && in_digit <= (unsigned)kListKeys) {
+            // collect the keys that carry the picked top digit; their order does not matter.
+            if (t == 0) s_fill = 0u;
+            __syncthreads();
+            // One block has the instruction throughput and the memory bandwidth of one compute unit
+            // (measured: about 50 GB/s, 7 us per 100 000 four-byte keys), so the scan is written
+            // for few instructions per key: a lane counts its hits in a 16-byte load, reserves room
+            // for them with one LDS atomic (only lanes with hits take part), and stores them.
+            constexpr int KV = 16 / (int)sizeof(key_t);  // keys per 16-byte load
+            constexpr int kLoads = 16;  // 16-byte loads in flight per lane: a round trip to memory per round
+            const Pack<key_t, KV>* kv = reinterpret_cast<const Pack<key_t, KV>*>(keys);
+            const int nfull = m / KV;
+            for (int v0 = 0; v0 < nfull; v0 += kFinishBlock * kLoads) {
+                Pack<key_t, KV> kk[kLoads];
+#pragma unroll
+                for (int q = 0; q < kLoads; ++q) {
+                    const int v = v0 + q * kFinishBlock + t;
+                    if (v < nfull) {
+                        kk[q] = kv[v];
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < KV; ++c) kk[q].x[c] = ~prefix;  // never matches
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < kLoads; ++q) {
+                    unsigned hits = 0;
+#pragma unroll
+                    for (int c = 0; c < KV; ++c) hits += ((kk[q].x[c] & mask) == prefix) ? 1u : 0u;
+                    if (hits) {
+                        unsigned at = atomicAdd(&s_fill, hits);
+#pragma unroll
+                        for (int c = 0; c < KV; ++c)
+                            if ((kk[q].x[c] & mask) == prefix) s_list[at++] = kk[q].x[c];
+                    }
+                }
+            }
+            for (int i = nfull * KV + t; i < m; i += kFinishBlock) {  // fewer than KV keys
+                const key_t k1 = keys[i];
+                if ((k1 & mask) == prefix) s_list[atomicAdd(&s_fill, 1u)] = k1;
+            }
+            __syncthreads();
+            listed = s_fill;
+            }
+        __syncthreads();
     }
     if (t == 0) {
         T v = value_of(prefix, T());
@@ -459,14 +534,26 @@ void dispatch_hist(cx_handle h, int smode, bool vec_ok, const T* vec, const T* a
     }
 }
 
+// Shift and width of radix pass p of a key of Elem<T>::key_bits bits.
+template <typename T> void pass_digits(int p, int* shift, int* bits, int* last) {
+    constexpr int kKeyBits = Elem<T>::key_bits;
+    constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
+    *shift = kKeyBits - kRadixBits * (p + 1);
+    *bits = kRadixBits;
+    if (*shift < 0) {
+        *bits += *shift;
+        *shift = 0;
+    }
+    *last = p == kPasses - 1 ? 1 : 0;
+}
+
 }  // namespace
 
 // The key of descending rank `rank` among the m keys described by (vec, add_vec, d_idx, mode).
 template <typename T>
 int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
                 float stepsize, unsigned long long rank, int plus_one, T* d_thr_out) {
-    constexpr int kKeyBits = Elem<T>::key_bits;
-    constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     using key_t = typename Elem<T>::key_t;
 
     if (m <= kSmallSelect) {
@@ -480,12 +567,10 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
             h->sel_keys_bytes = bytes;
         }
         key_t* keys = static_cast<key_t*>(h->sel_keys);
-        const int shift0 = kKeyBits - kRadixBits;
-        int blocks = (m + kBlock - 1) / kBlock;
-        if (blocks > 2048) blocks = 2048;
-#define CX_FIRST(SM, HA)                                                                                          \
-    hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kBlock), 0, h->stream, vec, add_vec, d_idx, \
-                       m, n, stepsize, keys, h->sel, shift0, kRadixBits)
+        const int blocks = (m + kFinishBlock - 1) / kFinishBlock;
+#define CX_FIRST(SM, HA)                                                                                              \
+    hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kFinishBlock), 0, h->stream, vec, add_vec, \
+                       d_idx, m, n, stepsize, keys, h->sel)
         if (add_vec) {
             if (sample_mode == kSampleFull) CX_FIRST(0, true);
             else if (sample_mode == kSampleStrided) CX_FIRST(1, true);
@@ -506,18 +591,14 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
         ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
     hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank);
     for (int p = 0; p < kPasses; ++p) {
-        int shift = kKeyBits - kRadixBits * (p + 1);
-        int bits = kRadixBits;
-        if (shift < 0) {
-            bits += shift;
-            shift = 0;
-        }
+        int shift, bits, last;
+        pass_digits<T>(p, &shift, &bits, &last);
         if (add_vec)
             dispatch_hist<T, true>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, shift, bits);
         else
             dispatch_hist<T, false>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, shift, bits);
-        hipLaunchKernelGGL(select_pick_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, shift, bits,
-                           p == kPasses - 1 ? 1 : 0, plus_one, d_thr_out);
+        hipLaunchKernelGGL(select_pick_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, shift, bits, last,
+                           plus_one, d_thr_out);
     }
     CX_HIP(hipGetLastError());
     return CX_OK;
@@ -584,6 +665,91 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
 
 template <typename T>
 int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
+                          float stepsize, float topK, T* d_thr_out);
+
+// Exact whole-vector top-k threshold and the fused compress in ONE pass over both vectors:
+//   1. a strided sample gives a lower bound L of the threshold (as in select_rank_bracketed);
+//   2. one streaming pass does update += data and lists every |update| > L as a candidate pair,
+//      ascending, WITHOUT clearing anything;
+//   3. the threshold t >= L is the wanted order statistic among the candidates' magnitudes;
+//   4. the candidates above t are copied to the message and cleared in the residual.
+// The list is unusable when it holds too few candidates (L too high: ties, a freak sample) or
+// more than its capacity; the device notices, step 4 does nothing, and since step 2 left the
+// complete sum in `update` the answer comes from update alone: whole-vector selection on it and
+// the update-only compress.  Same bits either way.  One host synchronisation, at the end.
+template <typename T>
+int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
+                         float topK, T* d_thr_out, int* d_size_prefix) {
+    if (!d_thr_out) d_thr_out = static_cast<T*>(h->d_thr);
+    h->fused_topk_taken = 0;
+    constexpr int kSample = 1 << 16;
+    constexpr int PW = Elem<T>::pair_words;
+    const int pos = n > 0 ? cx_topk_pos((size_t)n, topK) : 0;
+    unsigned long long rank = pos > 0 ? (unsigned long long)pos : 0ull;
+    if (n > 0 && rank > (unsigned long long)(n - 1)) rank = (unsigned long long)(n - 1);
+    const double expect = n > 0 ? (double)(rank + 1) / (double)n * kSample : 0.0;
+    const unsigned long long sample_rank = (unsigned long long)(expect + 8.0 * std::sqrt(expect) + 8.0);
+    const bool vec_ok = ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(update)) & 15u) == 0;
+    const bool msg_ok = out_msg && (reinterpret_cast<uintptr_t>(out_msg) & 3u) == 0 && out_capacity >= 8;
+    const bool single_pass = h->fused_topk && data && update && n >= (1 << 23) && pos > 0 && vec_ok && msg_ok &&
+                             sample_rank < (unsigned long long)kSample / 16;
+    if (!single_pass) {
+        int rc = launch_topk_threshold<T>(h, update, data, n, nullptr, n, kSampleFull, 1.0f, topK, d_thr_out);
+        if (rc != CX_OK) return rc;
+        return launch_compact<T>(h, out_msg, out_capacity, data, update, n, nullptr, d_thr_out, d_size_prefix);
+    }
+
+    const size_t cap = (size_t)n / 16 > ((size_t)1 << 22) ? (size_t)n / 16 : ((size_t)1 << 22);
+    const size_t need = 8 + cap * PW * 4;
+    if (need > h->cand_bytes) {
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->cand) CX_HIP(hipFree(h->cand));
+        h->cand = nullptr;
+        h->cand_bytes = 0;
+        CX_HIP(hipMalloc(&h->cand, need + 256));
+        h->cand_bytes = need;
+    }
+    unsigned* cand_words = static_cast<unsigned*>(h->cand);
+    T* d_bound = reinterpret_cast<T*>(static_cast<char*>(h->d_thr) + 64);
+    unsigned* d_result = reinterpret_cast<unsigned*>(static_cast<char*>(h->d_thr) + 128);
+
+    // 1. lower bound
+    int rc = select_rank<T>(h, update, data, n, nullptr, kSample, kSampleStrided, (float)n / (float)kSample, sample_rank,
+                            0, d_bound);
+    if (rc != CX_OK) return rc;
+    // 2. accumulate + candidates
+    rc = launch_candidates<T>(h, cand_words, (long long)cap, data, update, n, d_bound);
+    if (rc != CX_OK) return rc;
+    // 3. threshold among the candidates
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
+    hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank);
+    for (int p = 0; p < kPasses; ++p) {
+        int shift, bits, last;
+        pass_digits<T>(p, &shift, &bits, &last);
+        hipLaunchKernelGGL(select_hist_pairs_kernel<T>, dim3(256), dim3(kBlock), 0, h->stream, cand_words, (unsigned)cap,
+                           h->sel, shift, bits);
+        hipLaunchKernelGGL(select_pick_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, shift, bits, last, 0,
+                           d_thr_out);
+    }
+    CX_HIP(hipGetLastError());
+    // 4. message + residual
+    rc = launch_filter<T>(h, cand_words, (unsigned)cap, rank, d_thr_out, update, n, static_cast<unsigned*>(out_msg),
+                          (out_capacity - 8) / (4 * PW), d_size_prefix, d_result);
+    if (rc != CX_OK) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 12, d_result, 2 * sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
+    CX_HIP(hipStreamSynchronize(h->stream));
+    h->fused_topk_taken = 1;
+    if (h->h_pinned[12] == 0) return CX_OK;
+
+    // change of plan: `update` holds the complete sum, the message has not been touched
+    h->fused_topk_taken = 2;
+    rc = select_rank<T>(h, update, nullptr, n, nullptr, n, kSampleFull, 1.0f, rank, 0, d_thr_out);
+    if (rc != CX_OK) return rc;
+    return launch_compact<T>(h, out_msg, out_capacity, nullptr, update, n, nullptr, d_thr_out, d_size_prefix);
+}
+
+template <typename T>
+int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
                           float stepsize, float topK, T* d_thr_out) {
     if (!d_thr_out) d_thr_out = static_cast<T*>(h->d_thr);
     if (m <= 0) {
@@ -607,5 +773,8 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
 template int launch_topk_threshold<float>(cx_handle, const float*, const float*, int, const int*, int, int, float, float, float*);
 template int launch_topk_threshold<double>(cx_handle, const double*, const double*, int, const int*, int, int, float, float, double*);
 template int launch_topk_threshold<int>(cx_handle, const int*, const int*, int, const int*, int, int, float, float, int*);
+template int launch_compress_topk<float>(cx_handle, void*, long long, const float*, float*, int, float, float*, int*);
+template int launch_compress_topk<double>(cx_handle, void*, long long, const double*, double*, int, float, double*, int*);
+template int launch_compress_topk<int>(cx_handle, void*, long long, const int*, int*, int, float, int*, int*);
 
 }  // namespace cx

@@ -118,6 +118,23 @@ class Handle:
             C.byref(nbytes) if sync else None))
         return nbytes.value if sync else None
 
+    def compress_topk(self, out_msg, data, update, topk, d_thr=None, size_prefix=None):
+        """Whole-vector ThresholdTopK(topk) on update + data and compress_add_update in one call
+        (a single pass over the vectors when they are large).  The threshold is left in d_thr
+        (1-element device tensor) or the handle's slot.  Returns bytes written."""
+        if data.numel() != update.numel():
+            raise ComprexError(_lib.CX_ERR_SIZE_MISMATCH, "vector sizes must be the same!")
+        nbytes = C.c_int(0)
+        check(self.lib.cx_ip_compress_topk(
+            self._h, _dt(update), _p(out_msg), out_msg.numel() * out_msg.element_size(), _p(data), _p(update),
+            update.numel(), float(topk), _p(d_thr), _p(size_prefix), C.byref(nbytes)))
+        return nbytes.value
+
+    def get_option(self, key):
+        v = C.c_int(0)
+        check(self.lib.cx_get_option(self._h, key.encode(), C.byref(v)))
+        return v.value
+
     def decompress(self, out, msg, sync=True):
         nbytes = C.c_int(0)
         check(self.lib.cx_ip_decompress(self._h, _dt(out), _p(out), out.numel(), _p(msg),

@@ -79,6 +79,19 @@ protected:
                                     thr, send_sizeBytes ? reinterpret_cast<int*>(src_address() + at) : nullptr, false);
     }
 
+    // residual += d_data with the entries above the threshold compressed into the message at
+    // `d_target`: one fused call when the threshold is a whole-vector top-k and the compressor
+    // has a path for it, else false (nothing done) and the caller takes the two steps.
+    bool fused_topk_into(void* d_target, long long capacity, const VarTYPE* d_data, int n, int* d_size_prefix) {
+        float topK = 0;
+        if (n != rests_size || n <= 0 || !threshold->whole_vector_topk(n, &topK)) return false;
+        if (topK > 1.0f || topK < 0.0f) return false;  // let prepare_with report it
+        // a claim without a fused call is harmless: the caller's prepare_with follows and overwrites it
+        VarTYPE* slot = threshold->claim_device_threshold();
+        if (!slot) return false;
+        return compressor->compress_topk_device(d_target, capacity, d_data, rests(), n, topK, slot, d_size_prefix);
+    }
+
 public:
     ComprEx()
         : compressor(new CompressorNone<VarTYPE>()), threshold(new ThresholdNone<VarTYPE>()), gaspiCxx_segment(NULL),
@@ -191,6 +204,16 @@ public:
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
+        float topK = 0;
+        if (size == rests_size && threshold->whole_vector_topk(size, &topK)) {
+            wait_for_room();
+            const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
+            if (fused_topk_into(src_address() + offset, bufferSize - offset, v.get(), size,
+                                send_sizeBytes ? reinterpret_cast<int*>(src_address()) : nullptr)) {
+                srcBuff_data->post();
+                return;
+            }
+        }
         threshold->prepare_with(rests(), rests_size, v.get(), size);
         if (size != rests_size) {
             char msg[100];
@@ -420,6 +443,10 @@ public:
         }
         send_half(so);  // the message of the previous call
         cxx::Staged<const VarTYPE> v(h, this->stage_, vector, (size_t)size, true, false);
+        if (this->fused_topk_into(half(wo), doublebuffer_offset, v.get(), size, nullptr)) {
+            update_doublebuffer_phase();
+            return;
+        }
         this->threshold->prepare_with(this->rests(), this->rests_size, v.get(), size);
         if (size != this->rests_size) {
             char msg[100];

@@ -80,8 +80,13 @@ int cx_synchronize(cx_handle h);
 /* Tuning switches: "compact_items" (16-byte loads per lane and tile: 2, 4 or 8),
  * "stage_alternate" (1 = every other compress walks the vector from its end, so that it starts on
  * what the previous one left in the memory-side cache), "profile_stage" (see cx_profile_read),
- * "reduce_variant".  Unknown keys return CX_ERR_INVALID. */
+ * "reduce_variant", "select_bracket" (1 = whole-vector thresholds try a one-pass selection first),
+ * "fused_topk" (1 = cx_ip_compress_topk may take its single-pass route).  Unknown keys return
+ * CX_ERR_INVALID. */
 int cx_set_option(cx_handle h, const char* key, int value);
+/* Reads an option back; also "fused_topk_taken": how the last cx_ip_compress_topk ran
+ * (0 = threshold and compress as two steps, 1 = single pass, 2 = single pass abandoned). */
+int cx_get_option(cx_handle h, const char* key, int* value);
 
 /* No counterpart in the reference: a measurement aid.  After cx_set_option(h, "profile_stage", 1)
  * every cx_ip_compress records a HIP event before and after its streaming kernel, on the handle's
@@ -132,6 +137,20 @@ int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capaci
                    const void* data, void* update, int n,
                    const void* thr_host, const void* d_thr,
                    int* d_size_prefix, int* h_bytes);
+
+/* ComprEx<T>::writeRemote with a whole-vector ThresholdTopK (src/comprEx.tpp:176-191 calling
+ * src/threshold.hxx:160-167 in its `n < subsamples` mode, :224-231, and src/compressor.hxx:44-51):
+ * the exact top-k threshold of |update + data| and the fused compress_add_update of
+ * cx_ip_compress, same message, residual and threshold as cx_topk_threshold followed by
+ * cx_ip_compress, but with ONE pass over the two vectors when n >= 2^23 and topK is small
+ * (a sampled lower bound of the threshold selects candidates during the accumulate pass; the
+ * exact threshold is found among them; if the bound turns out unusable the result is
+ * computed from the accumulated vector instead).  The threshold is left in `d_thr_out`
+ * (device T; NULL = the handle's slot).  Waits for the stream once.  Other arguments as
+ * cx_ip_compress. */
+int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity,
+                        const void* data, void* update, int n, float topK,
+                        void* d_thr_out, int* d_size_prefix, int* h_bytes);
 
 /* CompressorIndexPairs<T>::decompression_strategy (src/compressor.hxx:613-638): zero
  * all out_n elements, then out[index] = value.  A message whose n exceeds out_n leaves

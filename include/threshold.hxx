@@ -52,6 +52,12 @@ public:
     // Device address of the current threshold, or nullptr when only the host value exists.
     virtual const VarTYPE* device_threshold() { return nullptr; }
 
+    // Not in the reference.  True when prepare_with on n elements would apply the top-k rule to
+    // every element (no sub-sampling); the fraction is returned.  ComprEx then computes threshold
+    // and message in one fused call and leaves the threshold where claim_device_threshold() says.
+    virtual bool whole_vector_topk(int n, float* topK_out) const { return false; }
+    virtual VarTYPE* claim_device_threshold() { return nullptr; }
+
 protected:
     virtual bool is_aboveThreshold(const VarTYPE& target) = 0;
 
@@ -144,6 +150,19 @@ public:
 
     virtual const VarTYPE* device_threshold() {
         return on_device_ ? static_cast<const VarTYPE*>(cx_threshold_slot(this->handle_.get())) : nullptr;
+    }
+
+    // n < subsamples is the reference's test for using the whole vector (src/threshold.hxx:224-231)
+    virtual bool whole_vector_topk(int n, float* topK_out) const {
+        const int subsamples = cx_topk_subsamples(topK, default_subsamples, subsamples_factor);
+        if (topK_out) *topK_out = topK;
+        return subsamples < 0 || n < subsamples;
+    }
+    // the slot will hold the threshold once the caller's fused call has run
+    virtual VarTYPE* claim_device_threshold() {
+        on_device_ = true;
+        host_valid_ = false;
+        return static_cast<VarTYPE*>(cx_threshold_slot(this->handle_.get()));
     }
 
     virtual void prepare(const VarTYPE* vec, int vec_size) {

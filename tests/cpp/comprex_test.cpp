@@ -48,6 +48,54 @@ template <typename data_t> int comprex_p2p(const char* name) {
     return print_pass(errors);
 }
 
+// The same conservation gold on a vector large enough for the single-pass whole-vector top-k
+// (threshold and message from one pass over residual and data): ThresholdTopK with more
+// sub-samples than elements, integer-valued data so that every sum is exact.
+int comprex_p2p_large() {
+    typedef float data_t;
+    const int size = (1 << 23) + 3;
+    const int num_runs = 4;
+    std::vector<data_t> values(size), result(size, (data_t)0);
+    unsigned x = 12345u;
+    for (int i = 0; i < size; ++i) {
+        x = x * 1664525u + 1013904223u;
+        values[i] = (data_t)((int)((x >> 8) % 2000001u) - 1000000);
+    }
+    GaspiEnvironment env(1 << 30);
+    std::vector<ComprEx<data_t> > cmprex;
+    cmprex.reserve(2);
+    for (int rank = 0; rank < 2; ++rank) {
+        env.set_rank(rank, 2);
+        cmprex.emplace_back(env.get_segment(), size, 3.0f, true);
+        cmprex[rank].setThreshold(ThresholdTopK<data_t>(0.01f, 1 << 24));
+        cmprex[rank].setCompressor(CompressorIndexPairs<data_t>());
+        cmprex[rank].connectTo((rank + 1) % 2, (rank + 1) % 2, 3);
+    }
+    int errors = 0;
+    for (int run = 0; run < num_runs; ++run) {
+        if (run < num_runs - 1) cmprex[0].writeRemote(values.data(), size);
+        else cmprex[0].flushRests();
+        cmprex[1].readRemote_add(result.data(), size);
+        if (run == 0) {  // about one percent of the elements went out (ties at the threshold stay behind)
+            long sent = 0;
+            for (int i = 0; i < size; ++i) sent += result[i] != 0;
+            if (sent < size / 100 - 100 || sent > size / 100) {
+                std::cout << "first message carried " << sent << " elements" << std::endl;
+                ++errors;
+            }
+        }
+    }
+    for (int i = 0; i < size; ++i)
+        if (result[i] != (data_t)(num_runs - 1) * values[i]) {
+            if (errors < 5) std::cout << "Error in [" << i << "]: result: " << result[i] << std::endl;
+            ++errors;
+        }
+    std::vector<data_t> rests = cmprex[0].getRests();
+    for (auto e : rests) if (e != 0) ++errors;
+    std::cout << "ComprEx point to point, 8M elements, whole-vector top-k" << std::endl;
+    return print_pass(errors);
+}
+
 // Comprex_AllToOneAllreduce::apply / flush (reference src/allreduce.tpp:172-237), every rank's
 // part executed in the order the data dependencies impose.
 template <typename data_t> int all_to_one(const char* name, int numRanks, int size, int num_runs, float ratio) {
@@ -215,6 +263,7 @@ int main() {
     failed += comprex_p2p<int>("int");
     failed += comprex_p2p<float>("float");
     failed += comprex_p2p<double>("double");
+    failed += comprex_p2p_large();
     failed += all_to_one<int>("int", 4, 1000, 10, 0.01f);
     failed += all_to_one<float>("float", 3, 100000, 5, 0.001f);
     failed += variants_and_forwarders<int>("int");

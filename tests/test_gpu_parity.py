@@ -218,6 +218,96 @@ def test_exact_threshold_one_pass_bracket_and_fallbacks(dev, oracle, dtype):
         dev.set_option("select_bracket", 1)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_fused_exact_topk_single_pass_and_changes_of_plan(dev, oracle, dtype):
+    """cx_ip_compress_topk = whole-vector ThresholdTopK + compress_add_update.  Inputs that let the
+    single pass finish (route 1), inputs whose sampled bound is useless so that the answer is
+    recomputed from the accumulated vector (route 2: every magnitude equal, ties at the
+    threshold, small values exactly at the sampled positions), and parameters for which the
+    single pass is not attempted (route 0).  Message, residual and threshold: the checker's bits."""
+    rng = np.random.default_rng(23)
+    n = 9_000_001
+    ds = 1 << 24  # > n: whole-vector mode of the reference
+    if dtype == np.int32:
+        base = rng.integers(-100000, 100001, n).astype(np.int32)
+        add = rng.integers(-50, 51, n).astype(np.int32)
+        tie_vec = rng.integers(-9, 10, n).astype(np.int32)
+        big, small = (rng.integers(500, 1000, n).astype(np.int32), np.ones(65536, np.int32))
+    else:
+        base = (rng.standard_normal(n) * 3).astype(dtype)
+        add = (rng.standard_normal(n) * 0.1).astype(dtype)
+        tie_vec = np.round(rng.standard_normal(n) * 3).astype(dtype)
+        big, small = ((5 + rng.random(n)).astype(dtype), (rng.random(65536) * 1e-3).astype(dtype))
+    zero = np.zeros(n, dtype)
+    sample_pos = (np.arange(65536, dtype=np.float32) * (np.float32(n) / np.float32(65536))).astype(np.int64)
+    hostile = big.copy()
+    hostile[sample_pos] = small  # the strided sample only sees small values
+    cases = {
+        "random_p0.01": (base, add, 0.01, 1),
+        "random_p0.001": (base, add, 0.001, 1),
+        "random_p0.3": (base, add, 0.3, 0),
+        "all_equal": (np.full(n, 3, dtype), zero, 0.01, 2),
+        "ties_at_threshold": (tie_vec, zero, 0.02, 2 if dtype == np.int32 else None),
+        "small_at_sampled_positions": (hostile, zero, 0.01, 2),
+    }
+    thr_out = torch.zeros(1, dtype=NP2T[dtype], device="cuda")
+    try:
+        for name, (u, d, topk, route) in cases.items():
+            t = np.float32(topk)
+            want_thr = oracle.topk_prepare_with(u, d, t, ds, 10.0)
+            uu = u.copy()
+            want_msg = oracle.ip_compress(d.copy(), uu, want_thr)
+            for fused in (1, 0):
+                say("fused exact top-k", dtype.__name__, name, "fused_topk", fused)
+                dev.set_option("fused_topk", fused)
+                gu, gd = _gpu(u), _gpu(d)
+                buf = _msgbuf(n, dtype)
+                prefix = torch.zeros(1, dtype=torch.int32, device="cuda")
+                nbytes = dev.compress_topk(buf, gd, gu, t, d_thr=thr_out, size_prefix=prefix)
+                taken = dev.get_option("fused_topk_taken")
+                if fused and route is not None:
+                    assert taken == route, (name, taken)
+                if not fused:
+                    assert taken == 0
+                assert thr_out.cpu().numpy()[0] == want_thr, (name, taken)
+                assert nbytes == want_msg.size and int(prefix.item()) == nbytes, (name, nbytes, want_msg.size)
+                assert buf[:nbytes].cpu().numpy().tobytes() == want_msg.tobytes(), name
+                assert gu.cpu().numpy().tobytes() == uu.tobytes(), name
+                assert gd.cpu().numpy().tobytes() == d.tobytes(), name
+    finally:
+        dev.set_option("fused_topk", 1)
+
+
+def test_fused_exact_topk_message_buffer_too_small_and_bad_arguments(dev, oracle):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rng = np.random.default_rng(24)
+    n = (1 << 23) + 5
+    u, d = _rand(rng, n, np.float32), _rand(rng, n, np.float32, 0.3)
+    t = np.float32(0.01)
+    want_thr = oracle.topk_prepare_with(u, d, t, 1 << 24, 10.0)
+    uu = u.copy()
+    want_msg = oracle.ip_compress(d.copy(), uu, want_thr)
+    keep = 8 + 8 * 1000  # room for 1000 pairs
+    buf = torch.zeros(keep, dtype=torch.uint8, device="cuda")
+    gu, gd = _gpu(u), _gpu(d)
+    say("fused exact top-k, message buffer too small")
+    with pytest.raises(ComprexError) as e:
+        dev.compress_topk(buf, gd, gu, t)
+    assert e.value.code == _lib.CX_ERR_CAPACITY
+    assert dev.get_option("fused_topk_taken") == 1
+    got = buf.cpu().numpy()
+    assert got[:8].tobytes() == want_msg[:8].tobytes()          # header keeps the true count
+    assert got[8:].tobytes() == want_msg[8:keep].tobytes()      # the pairs that fit
+    assert gu.cpu().numpy().tobytes() == uu.tobytes()           # residual as after a full compress
+    with pytest.raises(ComprexError) as e:
+        dev.compress_topk(_msgbuf(n, np.float32), gd, gu, 1.5)
+    assert e.value.code == _lib.CX_ERR_TOPK
+    with pytest.raises(ComprexError) as e:
+        dev.compress_topk(_msgbuf(n, np.float32), gd[:-1], gu, 0.01)
+    assert e.value.code == _lib.CX_ERR_SIZE_MISMATCH
+
+
 def test_topk_threshold_indexed_and_device_slot(dev, oracle):
     rng = np.random.default_rng(15)
     n, m = 1_000_000, 10_000
