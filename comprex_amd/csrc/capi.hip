@@ -261,6 +261,8 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->reduce_variant = value;
     } else if (!strcmp(key, "fused_topk")) {
         h->fused_topk = value ? 1 : 0;
+    } else if (!strcmp(key, "select_short_list")) {
+        h->select_short_list = value ? 1 : 0;
     } else {
         return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     }
@@ -275,6 +277,7 @@ int cx_get_option(cx_handle h, const char* key, int* value) {
     else if (!strcmp(key, "select_bracket")) *value = h->select_bracket;
     else if (!strcmp(key, "reduce_variant")) *value = h->reduce_variant;
     else if (!strcmp(key, "fused_topk")) *value = h->fused_topk;
+    else if (!strcmp(key, "select_short_list")) *value = h->select_short_list;
     else if (!strcmp(key, "fused_topk_taken")) *value = h->fused_topk_taken;
     else return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     return CX_OK;

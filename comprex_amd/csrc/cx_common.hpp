@@ -54,6 +54,8 @@ struct SelectState {
     unsigned long long mask;       // which bits of `prefix` are fixed
     unsigned long long rank;       // descending rank still to find among matching keys
     unsigned int hist[kRadixBins]; // digit histogram of the current pass
+    unsigned int short_count;      // two-launch select: keys in the short list; zero between runs
+    unsigned int short_digit;      // ... and the largest digit a block cut its share at
 };
 
 // Device status word: first error wins.
@@ -102,6 +104,7 @@ struct cx_handle_s {
     int compact_items = 4;             // 16-byte loads per lane and tile
     int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
     int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound
+    int select_short_list = 1;         // 1 = the two-launch select passes a short list of top keys to its second launch
     int fused_topk = 1;                // 1 = cx_ip_compress_topk may take its single-pass route
     int fused_topk_taken = 0;          // how the last cx_ip_compress_topk ran: 0 two calls, 1 single pass, 2 single pass abandoned
     int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter

@@ -262,15 +262,22 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
 // when the keys sharing the picked top digit fit in LDS they are collected there in one scan of
 // `keys` and the other passes never leave LDS, else every pass scans `keys` again.
 constexpr int kFinishBlock = 1024;
+constexpr int kShortListBytes = 32768;  // LDS list of the second launch, and the first launch's short list
 
 template <typename T, int SMODE, bool HAS_ADD>
 __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                               const int* __restrict__ idx, int m, int n, float stepsize,
                                                               typename Elem<T>::key_t* __restrict__ keys,
-                                                              SelectState* __restrict__ st) {
+                                                              SelectState* __restrict__ st, int short_k,
+                                                              typename Elem<T>::key_t* __restrict__ short_keys,
+                                                              unsigned short_cap) {
     using key_t = typename Elem<T>::key_t;
     constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
     __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit, s_base, s_wave[kFinishBlock / 64];
+    __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
+    key_t mine = 0;       // with short_k > 0 the grid covers m: one key per thread
+    bool have = false;
     // large blocks: every block ends with one global atomic per digit it has seen, and those
     // queue up per address
     for (int b = threadIdx.x; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
@@ -298,21 +305,51 @@ __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __r
             if (HAS_ADD) v = (T)(v + add[p]);
             k = ok ? key_of(v) : (key_t)0;
             keys[i] = k;
+            mine = k;
+            have = true;
         }
         hist_add(lds_hist, i < m, (unsigned)(k >> shift0) & ((1u << kRadixBits) - 1u));
     }
     merge_hist<kFinishBlock>(lds_hist, st);
+    if (short_k <= 0) return;
+
+    // Short list: the single-block second launch is bound by how many keys it must read, and
+    // the key it looks for is near the top.  Each block passes on only its keys from the top
+    // digit of its own short_k-th largest key upwards (all its keys when it has fewer), and the
+    // largest such digit over all blocks is recorded.  If the digit the second launch picks is
+    // not below that, every key carrying it is in the short list, and the full key array is not
+    // needed.
+    unsigned digit;
+    unsigned long long above;
+    block_pick<kFinishBlock>(lds_hist, (unsigned long long)(short_k - 1), s_sum, &s_digit, &s_above, digit, above);
+    const unsigned my_digit = (unsigned)(mine >> shift0) & ((1u << kRadixBits) - 1u);
+    const bool out = have && my_digit >= digit;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned long long votes = __ballot(out);
+    if (lane == 0) s_wave[wave] = (unsigned)__popcll(votes);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned total = 0;
+        for (int w = 0; w < kFinishBlock / 64; ++w) total += s_wave[w];
+        s_base = atomicAdd(&st->short_count, total);
+        atomicMax(&st->short_digit, digit);
+    }
+    __syncthreads();
+    unsigned at = s_base + (unsigned)__popcll(votes & (lane == 0 ? 0ull : (~0ull >> (64 - lane))));
+    for (int w = 0; w < wave; ++w) at += s_wave[w];
+    if (out && at < short_cap) short_keys[at] = mine;  // an overflowing list is seen from its count
 }
 
 template <typename T>
 __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typename Elem<T>::key_t* __restrict__ keys,
                                                                      int m, SelectState* __restrict__ st,
                                                                      unsigned long long rank, int plus_one,
-                                                                     T* __restrict__ thr_out) {
+                                                                     T* __restrict__ thr_out, int short_on,
+                                                                     const typename Elem<T>::key_t* __restrict__ short_keys) {
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
-    constexpr int kListKeys = 32768 / (int)sizeof(key_t);
+    constexpr int kListKeys = kShortListBytes / (int)sizeof(key_t);
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ key_t s_list[kListKeys];
     __shared__ unsigned s_digit, s_fill;
@@ -324,7 +361,14 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         lds_hist[b] = st->hist[b];
         st->hist[b] = 0u;  // leave it clean for the next run
     }
+    // what the first launch's blocks passed on
+    const unsigned short_count = short_on ? st->short_count : 0u;
+    const unsigned short_digit = short_on ? st->short_digit : 0u;
     __syncthreads();
+    if (short_on && t == 0) {  // clean for the next run
+        st->short_count = 0u;
+        st->short_digit = 0u;
+    }
     key_t prefix = 0, mask = 0;
     unsigned listed = 0;  // keys in s_list (0 = scan `keys`)
     for (int p = 0; p < kPasses; ++p) {
@@ -358,7 +402,17 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         prefix |= (key_t)digit << shift;
         mask |= (key_t)((1ull << bits) - 1ull) << shift;
         rank -= above;
-        if (p == 0 && in_digit <= (unsigned)kListKeys) {
+        if (p == 0 && short_on && short_count <= (unsigned)kListKeys && digit >= short_digit) {
+            // the short list holds every key with the picked top digit: keep those
+            if (t == 0) s_fill = 0u;
+            __syncthreads();
+            for (unsigned i = t; i < short_count; i += kFinishBlock) {
+                const key_t k1 = short_keys[i];
+                if ((k1 & mask) == prefix) s_list[atomicAdd(&s_fill, 1u)] = k1;
+            }
+            __syncthreads();
+            listed = s_fill;
+        } else if (p == 0 && in_digit <= (unsigned)kListKeys) {
             // collect the keys that carry the picked top digit; their order does not matter.
             if (t == 0) s_fill = 0u;
             __syncthreads();
@@ -563,14 +617,24 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
             h->sel_keys = nullptr;
             h->sel_keys_bytes = 0;
             size_t bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
-            CX_HIP(hipMalloc(&h->sel_keys, bytes));
+            CX_HIP(hipMalloc(&h->sel_keys, bytes + kShortListBytes));  // key array, then the short list
             h->sel_keys_bytes = bytes;
         }
         key_t* keys = static_cast<key_t*>(h->sel_keys);
+        key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) +
+                                                     (size_t)kSmallSelect * sizeof(unsigned long long));
         const int blocks = (m + kFinishBlock - 1) / kFinishBlock;
+        // short list: worth it when the wanted rank is near the top, so that a block's share of the
+        // keys above it (plus 8 sigma) is a small part of the block, and the shares fit the list
+        const unsigned short_cap = (unsigned)(kShortListBytes / (int)sizeof(key_t));
+        const double share = (double)(rank + 1) / (double)blocks;
+        int short_k = (int)(share + 8.0 * std::sqrt(share) + 8.0);
+        if (!h->select_short_list || m < 8192 || short_k > kFinishBlock / 4 ||
+            (double)blocks * (short_k + 16) > (double)short_cap)
+            short_k = 0;
 #define CX_FIRST(SM, HA)                                                                                              \
     hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kFinishBlock), 0, h->stream, vec, add_vec, \
-                       d_idx, m, n, stepsize, keys, h->sel)
+                       d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
         if (add_vec) {
             if (sample_mode == kSampleFull) CX_FIRST(0, true);
             else if (sample_mode == kSampleStrided) CX_FIRST(1, true);
@@ -582,7 +646,7 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
         }
 #undef CX_FIRST
         hipLaunchKernelGGL(select_finish_kernel<T>, dim3(1), dim3(kFinishBlock), 0, h->stream, keys, m, h->sel, rank,
-                           plus_one, d_thr_out);
+                           plus_one, d_thr_out, short_k > 0 ? 1 : 0, short_keys);
         CX_HIP(hipGetLastError());
         return CX_OK;
     }

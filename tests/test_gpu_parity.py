@@ -327,6 +327,42 @@ def test_topk_threshold_indexed_and_device_slot(dev, oracle):
     assert gv.cpu().numpy().tobytes() == uu.tobytes()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sampled_threshold_short_list_and_inputs_that_defeat_it(dev, oracle, dtype):
+    """The two-launch select hands its second launch a short list of each block's top keys and
+    falls back on the full key array when the list cannot hold the answer: large values
+    clustered in a few blocks' share of the samples, all-equal keys (list overflows), sample sets
+    too small or ranks too deep for the list.  Same threshold as the checker with the list on and off."""
+    rng = np.random.default_rng(31)
+    n = 3_000_000
+    if dtype == np.int32:
+        spread = rng.integers(-1_000_000, 1_000_001, n).astype(np.int32)
+        add = rng.integers(-10, 11, n).astype(np.int32)
+    else:
+        spread = (rng.laplace(size=n) * 2).astype(dtype)
+        add = (rng.standard_normal(n) * 0.05).astype(dtype)
+    clustered = (spread // 1000 if dtype == np.int32 else spread * 1e-3).astype(dtype)
+    clustered[: n // 40] = spread[: n // 40]            # every large value sits at the front
+    equal = np.full(n, 7, dtype)
+    zero = np.zeros(n, dtype)
+    try:
+        for name, v, a in [("spread", spread, add), ("clustered", clustered, zero), ("equal", equal, zero)]:
+            gv, ga = _gpu(v), _gpu(a)
+            for m, topk in [(100_000, 0.01), (65_536, 0.0133), (8_192, 0.01), (200_000, 0.002), (100_000, 0.2),
+                            (262_144, 0.01), (5_000, 0.01)]:
+                idx = np.sort(rng.integers(0, n, m)).astype(np.int32)
+                want = oracle.topk_prepare_indexed(v, a, idx, np.float32(topk))
+                gi = _gpu(idx)
+                for short in (1, 0):
+                    say("sampled threshold", dtype.__name__, name, m, topk, "short list", short)
+                    dev.set_option("select_short_list", short)
+                    assert dev.topk_threshold_indexed(gv, ga, gi, np.float32(topk)) == want
+                    # twice: the state the first run leaves must be clean
+                    assert dev.topk_threshold_indexed(gv, ga, gi, np.float32(topk)) == want
+    finally:
+        dev.set_option("select_short_list", 1)
+
+
 def test_topk_threshold_errors(dev):
     from comprex_amd.device import ComprexError
     from comprex_amd import _lib
