@@ -98,11 +98,18 @@ __device__ __forceinline__ void put_pair(unsigned* w, unsigned index, double v) 
     w[2] = (unsigned)(bits >> 32);
 }
 
+template <typename T> __device__ __forceinline__ T pair_value(const unsigned* w);
+template <> __device__ __forceinline__ float pair_value<float>(const unsigned* w) { return __uint_as_float(w[1]); }
+template <> __device__ __forceinline__ int pair_value<int>(const unsigned* w) { return (int)w[1]; }
+template <> __device__ __forceinline__ double pair_value<double>(const unsigned* w) {
+    return __longlong_as_double((long long)((unsigned long long)w[1] | ((unsigned long long)w[2] << 32)));
+}
+
 // One wavefront, one tile.  MODE 0: update += data, select on update, zero selected
 // (compress_add_update); MODE 1: select on update, zero selected (compress_update);
-// MODE 2: select on data, nothing written back (compress); MODE 3: update += data, select on
-// update, nothing zeroed (candidate pass of the fused exact top-k: the selected set is a superset
-// of what is finally sent, and the residual must survive a change of plan untouched).
+// MODE 2: select on data, nothing written back (compress); MODE 3: as MODE 0 for a list of
+// CANDIDATES (fused exact top-k: the selected set is a superset of what is finally sent): a
+// selected element that finds no room in the list is not an error, it keeps its value in update.
 // DIRECT false: stage the pairs (or defer the tile); true: write them at `direct_pos`.
 template <typename T, int MODE, int VEC, int ITEMS, bool DIRECT>
 __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* __restrict__ update, long long n,
@@ -130,7 +137,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         unsigned valid = (1u << VEC) - 1u;
         if (full) {
             if (MODE != 2) u = load_pack<T, VEC>(update + e0, false);
-            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);  // MODE 3 reads both
+            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
         } else {
             valid = 0;
 #pragma unroll
@@ -191,13 +198,14 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         Pack<T, VEC> w;
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
-            const bool keep = (m >> c) & 1u;
+            bool keep = (m >> c) & 1u;
             if (keep) {
                 if (pos < dst_limit) put_pair(dst + pos * PW, (unsigned)(e0 + c), s[j][c]);
+                else if (MODE == 3) keep = false;  // no room in the candidate list: stays in the residual
                 else overflow = true;
                 ++pos;
             }
-            w.x[c] = (keep && MODE != 3) ? (T)0 : s[j][c];
+            w.x[c] = keep ? (T)0 : s[j][c];
         }
         if (MODE != 2) {
             if (full) {
@@ -367,6 +375,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
                 if (dst_pos < cap_pairs) {
 #pragma unroll
                     for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
+                } else if (MODE == 3) {
+                    update[v[q][0]] = pair_value<T>(v[q]);  // no room in the candidate list: back into the residual
                 } else {
                     overflow = true;
                 }
@@ -472,9 +482,7 @@ int launch_mode(cx_handle h, int mode, const T* data, T* update, int n, const T*
     if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
     if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
     if (mode == 2) return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
-    // candidate pass: an overflowing candidate buffer is a change of plan, not an error of the caller
-    return launch_all<T, 3, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix,
-                                        reinterpret_cast<DeviceStatus*>(static_cast<char*>(h->d_thr) + 192));
+    return launch_all<T, 3, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
 }
 
 }  // namespace
@@ -512,8 +520,9 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
 }
 
 // ---- fused exact top-k: candidate pass and final filter -------------------------------------
-// Candidate pass: update += data (nothing zeroed) and every element with |update| > *d_bound as an
-// (index, value) pair, ascending, behind a message header in `cand_words`.
+// Candidate pass: update += data; every element with |update| > *d_bound leaves the residual for
+// the candidate list ((index, value) pairs, ascending, behind a message header in `cand_words`);
+// what the list has no room for stays in the residual, the header counts it all the same.
 template <typename T>
 int launch_candidates(cx_handle h, unsigned* cand_words, long long cap_pairs, const T* data, T* update, int n,
                       const T* d_bound) {
@@ -530,13 +539,6 @@ namespace {
 
 constexpr int kFilterBlocks = 2048;
 constexpr int kFilterBlock = 256;
-
-template <typename T> __device__ __forceinline__ T pair_value(const unsigned* w);
-template <> __device__ __forceinline__ float pair_value<float>(const unsigned* w) { return __uint_as_float(w[1]); }
-template <> __device__ __forceinline__ int pair_value<int>(const unsigned* w) { return (int)w[1]; }
-template <> __device__ __forceinline__ double pair_value<double>(const unsigned* w) {
-    return __longlong_as_double((long long)((unsigned long long)w[1] | ((unsigned long long)w[2] << 32)));
-}
 
 // The candidate list is usable when it holds the wanted order statistic (more candidates than
 // the rank) and nothing was dropped from it.
@@ -571,9 +573,10 @@ __global__ __launch_bounds__(kFilterBlock) void filter_count_kernel(const unsign
     if (threadIdx.x == 0) block_counts[blockIdx.x] = s_cnt;
 }
 
-// Copies the survivors to the message in list order and clears their residual entries; the last
-// block writes the header.  result[0]: 0 = done, 1 = candidate list not usable (nothing written);
-// result[1]: pairs in the message, or the candidate count.
+// Copies the survivors to the message in list order and gives the other candidates back to the
+// residual (the candidate pass cleared them all); the last block writes the header.  When the
+// list is not usable every listed candidate goes back and the message is not touched.
+// result[0]: 0 = done, 1 = list not usable; result[1]: pairs in the message, or the candidate count.
 template <typename T>
 __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
     const unsigned* __restrict__ cand_words, unsigned cand_cap, unsigned long long rank, const T* __restrict__ thr_ptr,
@@ -586,6 +589,11 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const unsigned count = cand_words[1];
     if (!candidates_usable(count, cand_cap, rank)) {
+        const unsigned listed = count < cand_cap ? count : cand_cap;
+        for (unsigned i = blockIdx.x * kFilterBlock + tid; i < listed; i += kFilterBlocks * kFilterBlock) {
+            const unsigned* w = cand_words + 2 + (size_t)i * PW;
+            if (w[0] < (unsigned)n) update[w[0]] = pair_value<T>(w);
+        }
         if (blockIdx.x == 0 && tid == 0) {
             result[0] = 1u;
             result[1] = count;
@@ -617,6 +625,7 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
 #pragma unroll
             for (int q = 0; q < PW; ++q) w[q] = cand_words[2 + (size_t)i * PW + q];
             keep = mag(pair_value<T>(w)) > thr;
+            if (!keep && w[0] < (unsigned)n) update[w[0]] = pair_value<T>(w);  // stays behind
         }
         const unsigned long long votes = __ballot(keep);
         if (lane == 0) s_wave[wave] = (unsigned)__popcll(votes);
@@ -635,7 +644,6 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
             } else {
                 overflow = true;
             }
-            if (w[0] < (unsigned)n) update[w[0]] = (T)0;
         }
         pos += all;
         __syncthreads();
@@ -652,8 +660,9 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
 
 }  // namespace
 
-// Final step of the fused exact top-k: the candidates above *d_thr become the message and leave
-// the residual; nothing happens (result[0] = 1) when the candidate list cannot hold the answer.
+// Final step of the fused exact top-k: the candidates above *d_thr become the message, the
+// others return to the residual; when the candidate list cannot hold the answer (result[0] = 1)
+// all of them return and the residual holds the complete sum again.
 template <typename T>
 int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, const T* d_thr,
                   T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result) {

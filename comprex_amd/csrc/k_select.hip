@@ -733,14 +733,15 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
 
 // Exact whole-vector top-k threshold and the fused compress in ONE pass over both vectors:
 //   1. a strided sample gives a lower bound L of the threshold (as in select_rank_bracketed);
-//   2. one streaming pass does update += data and lists every |update| > L as a candidate pair,
-//      ascending, WITHOUT clearing anything;
+//   2. one streaming pass does update += data and moves every |update| > L out of the residual
+//      into a list of candidate pairs, ascending (the fused compress with threshold L);
 //   3. the threshold t >= L is the wanted order statistic among the candidates' magnitudes;
-//   4. the candidates above t are copied to the message and cleared in the residual.
+//   4. the candidates above t are copied to the message, the others go back into the residual.
 // The list is unusable when it holds too few candidates (L too high: ties, a freak sample) or
-// more than its capacity; the device notices, step 4 does nothing, and since step 2 left the
-// complete sum in `update` the answer comes from update alone: whole-vector selection on it and
-// the update-only compress.  Same bits either way.  One host synchronisation, at the end.
+// not all of them (more than its capacity; the excess never left the residual); the device
+// notices, step 4 returns every listed candidate instead, and since `update` then holds the
+// complete sum the answer comes from update alone: whole-vector selection on it and the
+// update-only compress.  Same bits either way.  One host synchronisation, at the end.
 template <typename T>
 int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
                          float topK, T* d_thr_out, int* d_size_prefix) {
