@@ -48,6 +48,14 @@ template <> struct Elem<double> {
 constexpr int kRadixBits = 11;
 constexpr int kRadixBins = 1 << kRadixBits;
 
+// What is fixed of the wanted key after some passes.
+struct PickState {
+    unsigned long long prefix;     // key bits fixed so far
+    unsigned long long mask;       // which bits of `prefix` are fixed
+    unsigned long long rank;       // descending rank still to find among matching keys
+};
+constexpr int kMaxRadixPasses = 6; // 63-bit keys, 11 bits per pass
+
 // State of one radix-select run; lives in device memory.
 struct SelectState {
     unsigned long long prefix;     // key bits fixed so far
@@ -56,6 +64,10 @@ struct SelectState {
     unsigned int hist[kRadixBins]; // digit histogram of the current pass
     unsigned int short_count;      // two-launch select: keys in the short list; zero between runs
     unsigned int short_digit;      // ... and the largest digit a block cut its share at
+    // chained passes (no pick launch in between): one histogram per pass, all zero between runs,
+    // and the state entering each pass
+    unsigned int pass_hist[kMaxRadixPasses][kRadixBins];
+    PickState pass_state[kMaxRadixPasses];
 };
 
 // Device status word: first error wins.
@@ -126,7 +138,7 @@ template <typename T>
 int launch_candidates(cx_handle h, unsigned* cand_words, long long cap_pairs, const T* data, T* update, int n,
                       const T* d_bound);
 template <typename T>
-int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, const T* d_thr,
+int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, T* d_thr,
                   T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result);
 template <typename T>
 int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,

@@ -27,6 +27,7 @@
 // HBM traffic per element at low density (fp32): 4 B data + 4 B residual in, 4 B residual
 // out, plus per survivor 8 B staged + 8 B re-read + 8 B final.
 #include "cx_common.hpp"
+#include "cx_select_dev.hpp"
 
 namespace cx {
 
@@ -38,7 +39,10 @@ namespace {
 constexpr int kBlock = CX_STAGE_BLOCK;  // threads of a streaming block: one tile per wavefront
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
-constexpr int kGatherBlock = 256;  // tiles per gather block = tiles per group sum
+#ifndef CX_GATHER_BLOCK
+#define CX_GATHER_BLOCK 256
+#endif
+constexpr int kGatherBlock = CX_GATHER_BLOCK;  // tiles per gather block
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -298,7 +302,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
         // stage blocks before this block's first tile: kGatherBlock / kWavesPerBlock per gather block
         const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
         const unsigned nvec = blockIdx.x * (kGatherBlock / kWavesPerBlock / 4);
-#pragma unroll 4
+#pragma unroll 8
         for (unsigned v = tid; v < nvec; v += kGatherBlock) {
             const uint4 c = b4[v];
             before += c.x + c.y + c.z + c.w;
@@ -546,23 +550,31 @@ __device__ __forceinline__ bool candidates_usable(unsigned count, unsigned cap, 
     return (unsigned long long)count > rank && count <= cap;
 }
 
-// Survivors (|value| > threshold) per block-sized share of the candidate list.
+// Survivors (|value| > threshold) per block-sized share of the candidate list.  The threshold
+// is the key the chained radix passes over the candidates end on: every block does the last
+// pick itself from the last pass's histogram, block 0 stores the threshold for everyone after.
 template <typename T>
 __global__ __launch_bounds__(kFilterBlock) void filter_count_kernel(const unsigned* __restrict__ cand_words,
                                                                     unsigned cand_cap, unsigned long long rank,
-                                                                    const T* __restrict__ thr_ptr,
+                                                                    const SelectState* __restrict__ st,
+                                                                    T* __restrict__ thr_out,
                                                                     unsigned* __restrict__ block_counts) {
     constexpr int PW = Elem<T>::pair_words;
-    __shared__ unsigned s_cnt;
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
+    using key_t = typename Elem<T>::key_t;
+    __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_cnt, s_digit;
+    __shared__ unsigned long long s_above, s_sum[kFilterBlock / 64];
     if (threadIdx.x == 0) s_cnt = 0u;
-    __syncthreads();
+    const PickState done = state_entering_pass<T, kFilterBlock>(st, kPasses, rank, lds_hist, s_sum, &s_digit, &s_above);
+    const T thr = value_of((key_t)done.prefix, T());
+    if (blockIdx.x == 0 && threadIdx.x == 0) *thr_out = thr;
     const unsigned count = cand_words[1];
     unsigned mine = 0;
     if (candidates_usable(count, cand_cap, rank)) {
         const unsigned share = (count + kFilterBlocks - 1) / kFilterBlocks;
         const unsigned lo = blockIdx.x * share;
         const unsigned hi = lo + share < count ? lo + share : count;
-        const T thr = *thr_ptr;
         for (unsigned i = lo + threadIdx.x; i < hi; i += kFilterBlock)
             mine += mag(pair_value<T>(cand_words + 2 + (size_t)i * PW)) > thr ? 1u : 0u;
     }
@@ -581,12 +593,16 @@ template <typename T>
 __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
     const unsigned* __restrict__ cand_words, unsigned cand_cap, unsigned long long rank, const T* __restrict__ thr_ptr,
     const unsigned* __restrict__ block_counts, T* __restrict__ update, int n, unsigned* __restrict__ msg_words,
-    long long cap_pairs, int* __restrict__ size_prefix, unsigned* __restrict__ result, DeviceStatus* status) {
+    long long cap_pairs, int* __restrict__ size_prefix, unsigned* __restrict__ result, DeviceStatus* status,
+    SelectState* __restrict__ st) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kWaves = kFilterBlock / 64;
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     __shared__ unsigned s_before;
     __shared__ unsigned s_wave[kWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (blockIdx.x == 0)  // the chained passes' histograms have been read by everyone who needs them
+        for (int b = tid; b < kPasses * kRadixBins; b += kFilterBlock) (&st->pass_hist[0][0])[b] = 0u;
     const unsigned count = cand_words[1];
     if (!candidates_usable(count, cand_cap, rank)) {
         const unsigned listed = count < cand_cap ? count : cand_cap;
@@ -660,27 +676,28 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
 
 }  // namespace
 
-// Final step of the fused exact top-k: the candidates above *d_thr become the message, the
+// Final steps of the fused exact top-k: the threshold (last pick of the chained passes over the
+// candidates, left in *d_thr), then the candidates above it become the message, the
 // others return to the residual; when the candidate list cannot hold the answer (result[0] = 1)
 // all of them return and the residual holds the complete sum again.
 template <typename T>
-int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, const T* d_thr,
+int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, T* d_thr,
                   T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result) {
     // per-share counts live behind the per-block sums of the streaming pass, which are consumed by now
     int rc = ensure_scratch(h, (size_t)kFilterBlocks * kWavesPerBlock, 0);
     if (rc != CX_OK) return rc;
     hipLaunchKernelGGL(filter_count_kernel<T>, dim3(kFilterBlocks), dim3(kFilterBlock), 0, h->stream, cand_words,
-                       cand_cap, rank, d_thr, h->block_sums);
+                       cand_cap, rank, h->sel, d_thr, h->block_sums);
     hipLaunchKernelGGL(filter_write_kernel<T>, dim3(kFilterBlocks), dim3(kFilterBlock), 0, h->stream, cand_words,
                        cand_cap, rank, d_thr, h->block_sums, update, n, msg_words, cap_pairs, size_prefix, d_result,
-                       h->d_status);
+                       h->d_status, h->sel);
     CX_HIP(hipGetLastError());
     return CX_OK;
 }
 
 #define CX_INSTANTIATE_FUSED(T)                                                                                      \
     template int launch_candidates<T>(cx_handle, unsigned*, long long, const T*, T*, int, const T*);                 \
-    template int launch_filter<T>(cx_handle, const unsigned*, unsigned, unsigned long long, const T*, T*, int,       \
+    template int launch_filter<T>(cx_handle, const unsigned*, unsigned, unsigned long long, T*, T*, int,             \
                                   unsigned*, long long, int*, unsigned*);
 CX_INSTANTIATE_FUSED(float)
 CX_INSTANTIATE_FUSED(double)

@@ -14,6 +14,7 @@
 // second vector the key is |vec[p] + add_vec[p]| (one IEEE add, the same bits the
 // compressor's `update[i] += data[i]` produces later).
 #include "cx_common.hpp"
+#include "cx_select_dev.hpp"
 
 #include <cmath>
 
@@ -25,16 +26,6 @@ constexpr int kBlock = 256;
 constexpr int kSmallSelect = 1 << 18;  // sample sets up to this size take the two-launch path
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
-
-__device__ __forceinline__ uint32_t key_of(float v) { return __float_as_uint(v) & 0x7fffffffu; }
-__device__ __forceinline__ uint64_t key_of(double v) {
-    return (uint64_t)__double_as_longlong(v) & 0x7fffffffffffffffull;
-}
-__device__ __forceinline__ uint32_t key_of(int v) { return (uint32_t)(v < 0 ? -v : v); }
-
-__device__ __forceinline__ float value_of(uint32_t k, float) { return __uint_as_float(k); }
-__device__ __forceinline__ double value_of(uint64_t k, double) { return __longlong_as_double((long long)k); }
-__device__ __forceinline__ int value_of(uint32_t k, int) { return (int)k; }
 
 // ---- pieces shared by the selection kernels ------------------------------------------------
 // Digit count into an LDS histogram.  The keys a wavefront looks at together often share one
@@ -48,55 +39,6 @@ __device__ __forceinline__ void hist_add(unsigned* lds_hist, bool active, unsign
     const unsigned long long same = __ballot(active && digit == d0);
     if ((int)(threadIdx.x & 63) == leader) atomicAdd(&lds_hist[d0], (unsigned)__popcll(same));
     if (active && digit != d0) atomicAdd(&lds_hist[digit], 1u);
-}
-
-// Block-wide: digit holding descending rank `rank` in hist[0..kRadixBins), and how many keys
-// lie above that digit.  All threads get the result.  A rank beyond the total gives digit 0.
-template <int BLOCK>
-__device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long long rank, unsigned long long* s_sum,
-                                           unsigned* s_digit, unsigned long long* s_above, unsigned& digit,
-                                           unsigned long long& above) {
-    constexpr int kPer = kRadixBins / BLOCK;  // bins per thread
-    const int t = threadIdx.x;
-    const int hi = kRadixBins - 1 - t * kPer;  // thread t owns bins [hi - kPer + 1, hi], top digits first
-    unsigned cnt[kPer];
-    unsigned long long local = 0;
-#pragma unroll
-    for (int q = 0; q < kPer; ++q) {
-        cnt[q] = hist[hi - q];
-        local += cnt[q];
-    }
-    unsigned long long incl = local;  // inclusive scan over threads
-    const int lane = t & 63, wave = t >> 6;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const unsigned long long up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-    }
-    if (lane == 63) s_sum[wave] = incl;
-    if (t == 0) {
-        *s_digit = 0u;
-        *s_above = 0ull;
-    }
-    __syncthreads();
-    unsigned long long before = incl - local;
-    for (int w = 0; w < wave; ++w) before += s_sum[w];
-    if (rank >= before && rank < before + local) {
-        unsigned long long acc = before;
-#pragma unroll
-        for (int q = 0; q < kPer; ++q) {
-            if (rank < acc + cnt[q]) {
-                *s_digit = (unsigned)(hi - q);
-                *s_above = acc;
-                break;
-            }
-            acc += cnt[q];
-        }
-    }
-    __syncthreads();
-    digit = *s_digit;
-    above = *s_above;
-    __syncthreads();
 }
 
 __global__ __launch_bounds__(kBlock) void select_init_kernel(SelectState* st, unsigned long long rank) {
@@ -226,14 +168,27 @@ template <> __device__ __forceinline__ uint64_t pair_key<double>(const unsigned*
 
 template <typename T>
 __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigned* __restrict__ msg_words, unsigned cap,
-                                                                   SelectState* __restrict__ st, int shift, int bits) {
+                                                                   SelectState* __restrict__ st, int p,
+                                                                   unsigned long long rank0) {
     using key_t = typename Elem<T>::key_t;
     constexpr int PW = Elem<T>::pair_words;
     __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit;
+    __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    PickState s;
+    s.prefix = 0ull;
+    s.mask = 0ull;
+    s.rank = rank0;
+    if (p > 0) {
+        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above);
+        if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
+    }
     for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
     __syncthreads();
-    const key_t prefix = (key_t)st->prefix;
-    const key_t mask = (key_t)st->mask;
+    const key_t prefix = (key_t)s.prefix;
+    const key_t mask = (key_t)s.mask;
+    int shift, bits;
+    pass_digits_dev<T>(p, shift, bits);
     const unsigned digit_mask = (1u << bits) - 1u;
     unsigned m = msg_words[1];
     if (m > cap) m = cap;
@@ -253,7 +208,11 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
         for (int q = 0; q < 4; ++q)
             hist_add(lds_hist, in[q] && (k[q] & mask) == prefix, (unsigned)(k[q] >> shift) & digit_mask);
     }
-    merge_hist<kBlock>(lds_hist, st);
+    __syncthreads();
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+        const unsigned c = lds_hist[b];
+        if (c) atomicAdd(&st->pass_hist[p][b], c);
+    }
 }
 
 // ---- small sample sets: two launches ---------------------------------------------------
@@ -786,16 +745,12 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
     rc = launch_candidates<T>(h, cand_words, (long long)cap, data, update, n, d_bound);
     if (rc != CX_OK) return rc;
     // 3. threshold among the candidates
+    // (chained passes: the pick after each pass is redone by every block of the next kernel, the
+    // last one by the filter, which also writes the threshold and clears the histograms)
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
-    hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank);
-    for (int p = 0; p < kPasses; ++p) {
-        int shift, bits, last;
-        pass_digits<T>(p, &shift, &bits, &last);
+    for (int p = 0; p < kPasses; ++p)
         hipLaunchKernelGGL(select_hist_pairs_kernel<T>, dim3(256), dim3(kBlock), 0, h->stream, cand_words, (unsigned)cap,
-                           h->sel, shift, bits);
-        hipLaunchKernelGGL(select_pick_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, shift, bits, last, 0,
-                           d_thr_out);
-    }
+                           h->sel, p, rank);
     CX_HIP(hipGetLastError());
     // 4. message + residual
     rc = launch_filter<T>(h, cand_words, (unsigned)cap, rank, d_thr_out, update, n, static_cast<unsigned*>(out_msg),
