@@ -265,3 +265,47 @@ def test_optimizer_trains_over_simulated_ranks(schedule):
     assert not errors, errors
     for rank, (first, last) in losses.items():
         assert np.isfinite(last) and last < 0.7 * first, (schedule, rank, first, last)
+
+
+def test_sampled_step_can_be_captured_in_a_hip_graph():
+    """threshold (left on the device) + compress enqueue kernels only, so a caller may capture them.
+    Two steps (one in each walking direction) are captured and replayed three times, with eager
+    work and synchronisations in between; every replay gives the eager result."""
+    from comprex_amd.device import Handle, message_capacity
+    rng = np.random.default_rng(41)
+    n, m = 3_000_000, 20_000
+    g = torch.from_numpy(rng.laplace(size=n).astype(np.float32)).cuda()
+    idx = torch.from_numpy(rng.integers(0, n, m).astype(np.int32)).cuda()
+    rests = torch.zeros(n, device="cuda")
+    msg = torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        h = Handle()
+
+        def step():
+            h.topk_threshold_indexed(rests, g, idx, np.float32(0.01), to_host=False)
+            h.compress(msg, g, rests, sync=False)
+
+        for _ in range(2):  # scratch is allocated by now
+            step()
+        side.synchronize()
+        start = rests.clone()
+        step(), step()
+        side.synchronize()
+        want_rests = rests.clone()
+        want_msg = msg[: 8 + 8 * int(msg[4:8].view(torch.int32).item())].clone()
+        rests.copy_(start)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(), step()
+        side.synchronize()
+        for _ in range(3):
+            rests.copy_(start)
+            msg.zero_()
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            k = int(msg[4:8].view(torch.int32).item())
+            assert torch.equal(rests, want_rests)
+            assert torch.equal(msg[: 8 + 8 * k], want_msg)
+        h.synchronize()
