@@ -43,17 +43,26 @@ def _hex(x):
     return np.float32(x).tobytes().hex()
 
 
-def _error_feedback(dev, oracle, cfg, grad_fn, iters, gold_rows, oracle_live=True):
+def _error_feedback(dev, oracle, cfg, grad_fn, iters, gold_rows, oracle_live=True, fused_route=None):
+    """fused_route: None = threshold call then compress call; else the single call
+    (cx_ip_compress_topk) is used and must report that route."""
     n, topk, ds = cfg["n"], np.float32(cfg["topK"]), cfg["default_subsamples"]
     rests = torch.zeros(n, device="cuda")
     rests_h = np.zeros(n, np.float32)
     buf = _msgbuf(n)
+    thr_out = torch.zeros(1, device="cuda")
     compared = 0
     for it in range(iters):
         g_h = grad_fn(it)
         g = torch.from_numpy(g_h).cuda()
-        thr = dev.topk_threshold(rests, g, topk, ds)
-        nbytes = dev.compress(buf, g, rests)  # threshold from the handle's device slot
+        if fused_route is None:
+            thr = dev.topk_threshold(rests, g, topk, ds)
+            nbytes = dev.compress(buf, g, rests)  # threshold from the handle's device slot
+        else:
+            assert ds > n, "the single call is the whole-vector mode"
+            nbytes = dev.compress_topk(buf, g, rests, topk, d_thr=thr_out)
+            thr = float(thr_out.item())
+            assert dev.get_option("fused_topk_taken") == fused_route
         msg = buf[:nbytes].cpu().numpy()
         k = int(msg[4:8].view(np.int32)[0])
         say(cfg["name"], "iter", it, "thr", thr, "k", k)
@@ -80,6 +89,12 @@ def test_c1_one_million_top1pct_ten_iterations(dev, oracle):
 def test_c2_lenet5_top10pct_fifty_iterations(dev, oracle):
     compared = _error_feedback(dev, oracle, W.C2, W.c2_gradient, W.C2["iters"], GOLD["C2"])
     assert compared == W.C2["iters"]
+
+
+def test_c1_and_c3_threshold_and_compress_as_one_call(dev, oracle):
+    # C1 is too small for the single pass (route 0), C3 takes it (route 1); same recorded outputs
+    assert _error_feedback(dev, oracle, W.C1, W.c1_gradient, 3, GOLD["C1"], fused_route=0) == 3
+    assert _error_feedback(dev, oracle, W.C3, W.c3_gradient, 3, GOLD["C3"], fused_route=1) == 3
 
 
 def test_c3_resnet50_top0p1pct(dev, oracle):
@@ -119,6 +134,16 @@ def test_c4_hundred_million_laplace(dev, oracle):
     # reference-faithful strided sampling (1000 samples), exact top-k, and host-supplied positions
     run("strided", lambda r: dev.topk_threshold(r, g, topk, 1000, 10.0))
     run("exact", lambda r: dev.topk_threshold(r, g, topk, W.C4["default_subsamples_exact"], 10.0))
+    # the same as one call (single pass over the vectors): same recorded outputs
+    thr_out = torch.zeros(1, device="cuda")
+    r1 = torch.zeros(n, device="cuda")
+    nbytes = dev.compress_topk(buf, g, r1, topk, d_thr=thr_out)
+    assert dev.get_option("fused_topk_taken") == 1
+    row = GOLD["C4"]["exact"]
+    assert _hex(thr_out.item()) == row["thr_hex"] and nbytes == 8 + 8 * row["k"]
+    assert W.checksum(buf[:nbytes].cpu().numpy()) == row["msg"]
+    assert W.checksum(r1.cpu().numpy()) == row["rests"]
+    del r1
     idx_h = W.c4_sample_indices()
     assert W.checksum(idx_h) == GOLD["C4"]["indexed"]["idx"]
     idx = torch.from_numpy(idx_h).cuda()
