@@ -39,6 +39,9 @@ namespace {
 constexpr int kBlock = CX_STAGE_BLOCK;  // threads of a streaming block: one tile per wavefront
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
+#ifndef CX_GATHER_UNROLL
+#define CX_GATHER_UNROLL 8
+#endif
 #ifndef CX_GATHER_BLOCK
 #define CX_GATHER_BLOCK 256
 #endif
@@ -292,6 +295,9 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
     constexpr int kWaves = kGatherBlock / 64;
+    // pairs a lane moves per round: searches and loads of one round are independent, so a wavefront's
+    // whole share (about 64 tiles x 1 % x 1024 elements) is in flight at once
+    constexpr int kCopyUnroll = CX_GATHER_UNROLL;
     __shared__ unsigned s_before[kWaves];
     __shared__ unsigned s_wave_total[kWaves];
     __shared__ unsigned s_off[kWaves][65];
@@ -348,32 +354,31 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
 
     unsigned* const pairs = msg_words + 2;
     bool overflow = false;
-    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * 4) {
-        unsigned src_idx[4];
-        bool live[4];
+    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * kCopyUnroll) {
+        unsigned src_idx[kCopyUnroll];
+        bool live[kCopyUnroll];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < kCopyUnroll; ++q) {
             const unsigned p = p0 + q * 64 + lane;
             live[q] = p < wave_pairs;
-            // owner: last tile of this wavefront whose exclusive offset is <= p
-            int lo = 0, hi = 63;
-            while (lo < hi) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (so[mid] <= p) lo = mid;
-                else hi = mid - 1;
-            }
+            // owner: last tile of this wavefront whose exclusive offset is <= p.  Six fixed steps
+            // without branches, so that the searches of one round overlap their LDS reads.
+            int lo = 0;
+#pragma unroll
+            for (int step = 32; step > 0; step >>= 1)
+                lo += (so[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
             if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
             src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - so[lo]);
         }
-        unsigned v[4][PW];
+        unsigned v[kCopyUnroll][PW];
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < kCopyUnroll; ++q)
             if (live[q]) {
 #pragma unroll
                 for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
             }
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+        for (int q = 0; q < kCopyUnroll; ++q)
             if (live[q]) {
                 const long long dst_pos = (long long)wave_base + p0 + q * 64 + lane;
                 if (dst_pos < cap_pairs) {
