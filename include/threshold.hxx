@@ -121,18 +121,34 @@ template <class VarTYPE>
 class ThresholdTopK : public ThresholdFunction<VarTYPE> {
 public:
     ThresholdTopK(float topK, int default_subsamples = 1000, float subsample_factor = 10.0)
-        : _threshold(0), on_device_(false), host_valid_(true) {
+        : _threshold(0), on_device_(false), host_valid_(true), sample_m_(0) {
         if (topK > 1.0 || topK < 0.0) throw std::runtime_error("topK value must be between 0.0 and 1.0!");
         this->topK = topK;
         this->default_subsamples = default_subsamples;
         this->subsamples_factor = subsample_factor;
     }
 
-    // a clone carries the configuration and the last host-visible threshold, with scratch of its own
+    // a clone carries the configuration (sample positions included) and the last host-visible
+    // threshold, with scratch of its own
     ThresholdTopK(const ThresholdTopK<VarTYPE>& other)
         : topK(other.topK), default_subsamples(other.default_subsamples), subsamples_factor(other.subsamples_factor),
           _threshold(const_cast<ThresholdTopK<VarTYPE>&>(other).get_threshold()), on_device_(false),
-          host_valid_(true) {}
+          host_valid_(true), sample_m_(0) {
+        if (other.sample_m_ > 0) set_sample_positions(static_cast<const int*>(other.sample_idx_.data()), other.sample_m_);
+    }
+
+    // Not in the reference: prepare / prepare_with take the order statistic over these positions
+    // (int32 indices into the vector; host or device pointer, copied) instead of the strided
+    // sub-sample; m == 0 returns to the reference's rule.
+    void set_sample_positions(const int* idx, int m) {
+        sample_m_ = 0;
+        if (m <= 0) return;
+        if (!idx) throw std::runtime_error("sample positions: null pointer");
+        cx_handle h = this->handle_.get();
+        cxx::check(cx_copy(h, sample_idx_.reserve((size_t)m * sizeof(int)), idx, (size_t)m * sizeof(int)));
+        cxx::check(cx_synchronize(h));
+        sample_m_ = m;
+    }
 
     float getTopK() const { return topK; }
 
@@ -154,6 +170,7 @@ public:
 
     // n < subsamples is the reference's test for using the whole vector (src/threshold.hxx:224-231)
     virtual bool whole_vector_topk(int n, float* topK_out) const {
+        if (sample_m_ > 0) return false;
         const int subsamples = cx_topk_subsamples(topK, default_subsamples, subsamples_factor);
         if (topK_out) *topK_out = topK;
         return subsamples < 0 || n < subsamples;
@@ -166,6 +183,10 @@ public:
     }
 
     virtual void prepare(const VarTYPE* vec, int vec_size) {
+        if (sample_m_ > 0) {
+            prepare_indexed(vec, vec_size, nullptr, static_cast<const int*>(sample_idx_.data()), sample_m_);
+            return;
+        }
         cx_handle h = this->handle_.get();
         cxx::Staged<const VarTYPE> v(h, this->stage_in_, vec, (size_t)vec_size, true, false);
         cxx::check(cx_topk_threshold(h, cxx::dtype_of<VarTYPE>::value, v.get(), nullptr, vec_size, 0, topK,
@@ -176,6 +197,10 @@ public:
 
     virtual void prepare_with(const VarTYPE* vec, int vec_size, const VarTYPE* add_vec, int add_vec_size) {
         if (vec_size != add_vec_size) throw std::runtime_error("vector sizes must be the same!");
+        if (sample_m_ > 0) {
+            prepare_indexed(vec, vec_size, add_vec, static_cast<const int*>(sample_idx_.data()), sample_m_);
+            return;
+        }
         cx_handle h = this->handle_.get();
         cxx::Staged<const VarTYPE> v(h, this->stage_in_, vec, (size_t)vec_size, true, false);
         cxx::Staged<const VarTYPE> a(h, this->stage_hi_, add_vec, (size_t)add_vec_size, true, false);
@@ -204,6 +229,8 @@ protected:
     VarTYPE _threshold;
     bool on_device_;   // the handle's slot holds the current threshold
     bool host_valid_;  // _threshold mirrors it
+    cxx::DeviceBuffer sample_idx_;  // caller-chosen sample positions (device copy), sample_m_ of them
+    int sample_m_;
 
     virtual bool is_aboveThreshold(const VarTYPE& target) { return std::abs(target) >= get_threshold(); }
 };

@@ -2,6 +2,7 @@
 // library's ThresholdConst / ThresholdTopK, for int (as the reference) and float.
 #include <threshold.hxx>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <vector>
@@ -61,6 +62,47 @@ template <typename data_t> int run(const char* name) {
         try { ThresholdConst<data_t> t((data_t)-1); ++errors; } catch (const std::runtime_error&) {}
         ThresholdTopK<data_t> t(0.1f);
         try { t.prepare_with(values.data(), size, values.data(), size - 1); ++errors; } catch (const std::runtime_error&) {}
+        failed += print_pass(errors);
+    }
+    {  // caller-chosen sample positions: the order statistic of |v[p] + a[p]| over them, also in a clone
+        int errors = 0;
+        const int n = 5000, m = 700;
+        const float topK = 0.05f;
+        std::vector<data_t> v(n), a(n);
+        std::vector<int> pos(m);
+        unsigned x = 99u;
+        for (int i = 0; i < n; ++i) {
+            x = x * 1664525u + 1013904223u;
+            v[i] = (data_t)((int)((x >> 9) % 20001u) - 10000);
+            a[i] = (data_t)((int)((x >> 3) % 11u) - 5);
+        }
+        for (int i = 0; i < m; ++i) {
+            x = x * 1664525u + 1013904223u;
+            pos[i] = (int)((x >> 8) % (unsigned)n);
+        }
+        std::vector<data_t> mags(m);
+        for (int i = 0; i < m; ++i) mags[i] = (data_t)std::abs((data_t)(v[pos[i]] + a[pos[i]]));
+        std::sort(mags.begin(), mags.end(), [](data_t l, data_t r) { return l > r; });
+        const data_t gold = mags[(int)(std::ceil((float)m * topK) - 1.0f)];
+        ThresholdTopK<data_t> t(topK);
+        t.set_sample_positions(pos.data(), m);
+        t.prepare_with(v.data(), n, a.data(), n);
+        if (t.get_threshold() != gold) ++errors;
+        ThresholdFunction<data_t>* c = t.clone();
+        c->prepare_with(v.data(), n, a.data(), n);
+        if (c->get_threshold() != gold) ++errors;
+        delete c;
+        t.set_sample_positions(nullptr, 0);  // back to the strided rule: 1000 samples of 5000
+        t.prepare_with(v.data(), n, a.data(), n);
+        std::vector<data_t> strided(1000);
+        const float stepsize = (float)n / 1000.0f;
+        for (int i = 0; i < 1000; ++i) {
+            const int p = (int)((float)i * stepsize);
+            strided[i] = (data_t)std::abs((data_t)(v[p] + a[p]));
+        }
+        std::sort(strided.begin(), strided.end(), [](data_t l, data_t r) { return l > r; });
+        if (t.get_threshold() != strided[(int)(std::ceil(1000.0f * topK) - 1.0f)]) ++errors;
+        std::cout << "ThresholdTopK over caller-chosen positions (" << name << ")" << std::endl;
         failed += print_pass(errors);
     }
     return failed;
