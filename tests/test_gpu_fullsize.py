@@ -186,3 +186,62 @@ def test_c5_sparse_reduce_eight_ranks(dev, oracle):
     dev.add_vec(rests, torch.from_numpy(got).cuda())
     assert rests.cpu().numpy().tobytes() == want.tobytes()
     dev.synchronize()
+
+
+def test_largest_vector_an_int32_length_allows(dev):
+    """n = 2^31 - 1 elements (the reference's sizes are `int`): sampled threshold + fused compress,
+    the one-call exact top-k, and decompress, checked on the GPU against the definition
+    (k = #{|r+g| > t}, ascending indices = the positions of those elements, values = their sums,
+    residual = the sums with the sent ones cleared), chunk by chunk."""
+    n = 2**31 - 1
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    g = torch.empty(n, device="cuda").normal_(generator=gen)
+    r0 = torch.empty(n, device="cuda").normal_(std=0.25, generator=gen)
+    idx = torch.randint(0, n, (100_000,), device="cuda", dtype=torch.int32, generator=gen)
+    buf = torch.zeros(8 + 8 * (n // 50), dtype=torch.uint8, device="cuda")  # room for 2 %
+    chunks = [(a, min(a + (1 << 29), n)) for a in range(0, n, 1 << 29)]
+
+    def check(rests, thr, nbytes):
+        k = int(buf[4:8].view(torch.int32).item())
+        assert int(buf[0:4].view(torch.int32).item()) == n and nbytes == 8 + 8 * k
+        pairs = buf[8:nbytes].view(torch.int32).view(-1, 2)
+        got_idx, got_val = pairs[:, 0].long(), pairs[:, 1].contiguous().view(torch.float32)
+        at = 0
+        for a, b in chunks:
+            s = r0[a:b] + g[a:b]
+            sel = s.abs() > thr
+            pos = sel.nonzero().flatten()
+            c = pos.numel()
+            assert torch.equal(got_idx[at:at + c], pos + a)
+            assert torch.equal(got_val[at:at + c], s[pos])
+            assert torch.equal(rests[a:b], torch.where(sel, torch.zeros_like(s), s))
+            at += c
+            del s, sel, pos
+        assert at == k
+        return k
+
+    say("largest vector: sampled threshold + compress")
+    rests = r0.clone()
+    thr = dev.topk_threshold_indexed(rests, g, idx, np.float32(0.01))
+    nbytes = dev.compress(buf, g, rests)
+    k = check(rests, thr, nbytes)
+    assert abs(k / n - 0.01) < 0.002
+
+    say("largest vector: decompress")
+    dense = torch.empty(n, device="cuda")
+    assert dev.decompress(dense, buf) == nbytes
+    for a, b in chunks:
+        s = r0[a:b] + g[a:b]
+        assert torch.equal(dense[a:b], torch.where(s.abs() > thr, s, torch.zeros_like(s)))
+        del s
+    del dense
+
+    say("largest vector: threshold and compress as one call")
+    rests.copy_(r0)
+    thr_out = torch.zeros(1, device="cuda")
+    nbytes = dev.compress_topk(buf, g, rests, np.float32(0.01), d_thr=thr_out)
+    assert dev.get_option("fused_topk_taken") == 1
+    k = check(rests, float(thr_out.item()), nbytes)
+    # whole-vector top-k: the (pos+1)-th largest magnitude is the threshold, pos = ceil_f32(n*topK) - 1
+    pos = int(np.ceil(np.float32(n) * np.float32(0.01)) - np.float32(1.0))
+    assert pos - 8 <= k <= pos  # ties with the threshold stay behind
