@@ -60,6 +60,9 @@ def lib():
         "cx_ip_compress": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp, C.POINTER(i)]),
         "cx_ip_compress_topk": (i, [vp, i, vp, ll, vp, vp, i, C.c_float, vp, vp, C.POINTER(i)]),
         "cx_get_option": (i, [vp, C.c_char_p, C.POINTER(i)]),
+        "cx_rle_compress": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp, C.POINTER(i)]),
+        "cx_rle_decompress": (i, [vp, i, vp, i, vp, C.POINTER(i)]),
+        "cx_rle_add": (i, [vp, i, vp, i, vp]),
         "cx_ip_decompress": (i, [vp, i, vp, i, vp, C.POINTER(i)]),
         "cx_ip_add": (i, [vp, i, vp, i, vp, i]),
         "cx_ip_reduce": (i, [vp, i, vp, i, C.POINTER(vp), i, i, i]),

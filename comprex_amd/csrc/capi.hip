@@ -119,6 +119,20 @@ int compress_topk_impl(cx_handle h, void* out_msg, long long out_capacity, const
 }
 
 template <typename T>
+int rle_compress_impl(cx_handle h, void* out_msg, long long out_capacity, const void* data, void* update, int n,
+                      const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
+    int* d_result = reinterpret_cast<int*>(static_cast<char*>(h->d_thr) + 128);
+    int rc = launch_rle_compress<T>(h, out_msg, out_capacity, static_cast<const T*>(data), static_cast<T*>(update), n,
+                                    static_cast<const T*>(thr_host), static_cast<const T*>(d_thr), d_size_prefix,
+                                    d_result);
+    if (rc != CX_OK || !h_bytes) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, d_result, 4, hipMemcpyDeviceToHost, h->stream));
+    rc = collect_status(h);
+    *h_bytes = h->h_pinned[8];
+    return rc;
+}
+
+template <typename T>
 int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_bytes) {
     int rc = launch_decompress<T>(h, static_cast<T*>(out), out_n, msg);
     if (rc != CX_OK || !h_bytes) return rc;
@@ -216,6 +230,8 @@ int cx_destroy(cx_handle h) {
     if (h->sel) (void)hipFree(h->sel);
     if (h->sel_keys) (void)hipFree(h->sel_keys);
     if (h->cand) (void)hipFree(h->cand);
+    if (h->rle_pairs) (void)hipFree(h->rle_pairs);
+    if (h->rle_scan) (void)hipFree(h->rle_scan);
     if (h->d_status) (void)hipFree(h->d_status);
     if (h->d_thr) (void)hipFree(h->d_thr);
     if (h->h_pinned) (void)hipHostFree(h->h_pinned);
@@ -351,6 +367,25 @@ int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_c
     if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
     CX_DISPATCH(dt, compress_topk_impl<T>(h, out_msg, out_capacity, data, update, n, topK, d_thr_out, d_size_prefix,
                                           h_bytes));
+}
+
+int cx_rle_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
+                    int n, const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, rle_compress_impl<T>(h, out_msg, out_capacity, data, update, n, thr_host, d_thr, d_size_prefix,
+                                         h_bytes));
+}
+
+int cx_rle_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_n) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (!aligned4(msg)) return fail(CX_ERR_INVALID, "message must be 4-byte aligned");
+    CX_DISPATCH(dt, launch_rle_decode<T>(h, static_cast<T*>(out), out_n, msg, 0, h_n));
+}
+
+int cx_rle_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (!msg || !aligned4(msg)) return fail(CX_ERR_INVALID, "message must be a 4-byte aligned device pointer");
+    CX_DISPATCH(dt, launch_rle_decode<T>(h, static_cast<T*>(out), out_n, msg, 1, nullptr));
 }
 
 int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes) {

@@ -102,6 +102,10 @@ struct cx_handle_s {
     size_t cand_bytes = 0;
     void* sel_keys = nullptr;          // gathered sample keys of the two-launch select
     size_t sel_keys_bytes = 0;
+    void* rle_pairs = nullptr;         // run-length codec: the (index, value) pairs its compress starts from
+    size_t rle_pairs_bytes = 0;
+    unsigned* rle_scan = nullptr;      // run-length codec: per-block counts / prefix sums over the runs
+    size_t rle_scan_bytes = 0;
     cx::DeviceStatus* d_status = nullptr;
     void* d_thr = nullptr;             // 8-byte threshold slot
     int* h_pinned = nullptr;           // 64-byte pinned read-back area
@@ -143,6 +147,12 @@ int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, un
 template <typename T>
 int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
                          float topK, T* d_thr_out, int* d_size_prefix);
+
+// run-length codec
+template <typename T>
+int launch_rle_compress(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
+                        const T* thr_host, const T* d_thr, int* d_size_prefix, int* d_result);
+template <typename T> int launch_rle_decode(cx_handle h, T* out, int out_n, const void* msg, int add, int* n_out);
 
 template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg);
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);

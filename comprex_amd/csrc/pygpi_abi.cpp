@@ -125,9 +125,11 @@ float ThresholdTopK_getThreshold(void* self) {
     return guarded_value<float>(0.0f, [&] { return static_cast<ThresholdTopK<data_t>*>(self)->get_threshold(); });
 }
 
-// ---- compressors (src/comprEx_C.cpp:76-87; the run-length codec is not provided) ----------
+// ---- compressors (src/comprEx_C.cpp:76-87) ----------------------------------------------------
 void* CompressorNone_new(void) { return new CompressorNone<data_t>(); }
 void CompressorNone_del(void* self) { delete static_cast<CompressorNone<data_t>*>(self); }
+void* CompressorRLE_new(void) { return new CompressorRLE<data_t>(); }
+void CompressorRLE_del(void* self) { delete static_cast<CompressorRLE<data_t>*>(self); }
 void* CompressorIndexPairs_new(void) { return new CompressorIndexPairs<data_t>(); }
 void CompressorIndexPairs_del(void* self) { delete static_cast<CompressorIndexPairs<data_t>*>(self); }
 

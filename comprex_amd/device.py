@@ -135,6 +135,34 @@ class Handle:
         check(self.lib.cx_get_option(self._h, key.encode(), C.byref(v)))
         return v.value
 
+    # ---- run-length codec -------------------------------------------------
+    def rle_compress(self, out_msg, data, update, thr=None, d_thr=None, size_prefix=None, sync=True):
+        """CompressorRLE: as compress(), but |x| >= thr is sent and the message carries values
+        and run lengths instead of (index, value) pairs.  Returns bytes written when sync."""
+        ref = data if data is not None else update
+        if ref is None:
+            raise ComprexError(_lib.CX_ERR_INVALID, "Compression needs a valid input vector!")
+        if data is not None and update is not None and data.numel() != update.numel():
+            raise ComprexError(_lib.CX_ERR_SIZE_MISMATCH,
+                               "Compressor: Update vector size (%d) is not equal data vector size (%d)!"
+                               % (update.numel(), data.numel()))
+        hthr = _CT[ref.dtype](thr) if thr is not None else None
+        nbytes = C.c_int(0)
+        check(self.lib.cx_rle_compress(
+            self._h, _DT[ref.dtype], _p(out_msg), out_msg.numel() * out_msg.element_size(), _p(data), _p(update),
+            ref.numel(), C.byref(hthr) if hthr is not None else None, _p(d_thr), _p(size_prefix),
+            C.byref(nbytes) if sync else None))
+        return nbytes.value if sync else None
+
+    def rle_decompress(self, out, msg):
+        """Returns the vector length the message carries (what the reference's decoder returns)."""
+        n = C.c_int(0)
+        check(self.lib.cx_rle_decompress(self._h, _dt(out), _p(out), out.numel(), _p(msg), C.byref(n)))
+        return n.value
+
+    def rle_add(self, out, msg):
+        check(self.lib.cx_rle_add(self._h, _dt(out), _p(out), out.numel(), _p(msg)))
+
     def decompress(self, out, msg, sync=True):
         nbytes = C.c_int(0)
         check(self.lib.cx_ip_decompress(self._h, _dt(out), _p(out), out.numel(), _p(msg),

@@ -34,6 +34,7 @@ _PROTOS = {
     "ThresholdTopK_getThreshold": (_f, [_vp]),
     "GaspiEnvironment_set_blocking": (None, [_vp, _i, C.c_double]),
     "CompressorNone_new": (_vp, []), "CompressorNone_del": (None, [_vp]),
+    "CompressorRLE_new": (_vp, []), "CompressorRLE_del": (None, [_vp]),
     "CompressorIndexPairs_new": (_vp, []), "CompressorIndexPairs_del": (None, [_vp]),
 }
 for _fam, _setup in (("Comprex_AllToOneAllreduce", [_vp, _i, _i, _i, _f, _f]),
@@ -221,6 +222,14 @@ class CompressorNone(Getable):
 
     def __del__(self):
         libcomprex().CompressorNone_del(self.obj)
+
+
+class CompressorRLE(Getable):
+    def __init__(self):
+        self.obj = libcomprex().CompressorRLE_new()
+
+    def __del__(self):
+        libcomprex().CompressorRLE_del(self.obj)
 
 
 class CompressorIndexPairs(Getable):

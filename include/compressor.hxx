@@ -6,7 +6,7 @@
 //   CompressorNone<T>        dense copy: int32 n, then n values (:83-151)
 //   CompressorIndexPairs<T>  int32 n, int32 k, k x (int32 index, T value), ascending index
 //                                                              (:538-661)
-// The reference's run-length codec (:158-532) is not provided.
+//   CompressorRLE<T>         run-length codec: values + alternating run lengths  (:158-532)
 //
 // Vectors and message buffers may be host or device pointers.  The reference's calls carry no
 // buffer capacity; like the reference, the buffer is trusted to hold the message
@@ -191,6 +191,98 @@ protected:
             throw std::runtime_error("Decompression vector size is bigger than output buffer!");
         cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
         cxx::check(cx_ip_add(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_in, 0));
+        o.flush();
+        cxx::check(cx_synchronize(h));
+    }
+};
+
+// ---------------------------------------------------------------------------------------
+// Run-length codec (reference src/compressor.hxx:158-532): int32 n, int32 c, c values, int32 runs,
+// int32 signum, run lengths; an element is sent when |x| >= threshold.  The sent values are
+// stored densely, as the reference's decoder expects (its encoder indexes them by vector
+// position, :238,277,316, and only decodes when every element is sent).  decompress returns the
+// vector length the message carries, as the reference's does (:469), not a byte count.
+template <class VarTYPE>
+class CompressorRLE : public Compressor<VarTYPE> {
+public:
+    CompressorRLE() {}
+    CompressorRLE(const CompressorRLE<VarTYPE>& other) : Compressor<VarTYPE>(other) {}
+    virtual Compressor<VarTYPE>* clone() const { return new CompressorRLE<VarTYPE>(*this); }
+
+    // n values, n + 1 run lengths at most
+    static long long max_message_bytes(int n) { return 16 + (long long)n * (long long)sizeof(VarTYPE) + 4ll * ((long long)n + 1); }
+
+    virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
+                                const VarTYPE* d_threshold, VarTYPE threshold, int* d_size_prefix, bool wait) {
+        if (!d_data && !d_update) throw std::runtime_error("Compression needs a valid input vector!");
+        int bytes = -1;
+        cxx::check(cx_rle_compress(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, d_target, capacity, d_data,
+                                   d_update, n, d_threshold ? nullptr : &threshold, d_threshold, d_size_prefix,
+                                   wait ? &bytes : nullptr));
+        return bytes;
+    }
+    virtual int decompress_device(VarTYPE* d_output, int output_size, const void* d_source, bool) {
+        int n = 0;
+        const int rc = cx_rle_decompress(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, d_output, output_size,
+                                         d_source, &n);
+        if (rc == CX_ERR_MSG_TOO_LARGE) throw std::runtime_error("Decompression vector size is bigger than output buffer!");
+        cxx::check(rc);
+        return n;
+    }
+    virtual void add_device(VarTYPE* d_output, int output_size, const void* d_source) {
+        const int rc = cx_rle_add(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, d_output, output_size, d_source);
+        if (rc == CX_ERR_MSG_TOO_LARGE) throw std::runtime_error("Decompression vector size is bigger than output buffer!");
+        cxx::check(rc);
+    }
+
+protected:
+    virtual int compression_strategy(void* output, const VarTYPE* data_vector, VarTYPE* update_vector,
+                                     const int vector_size, VarTYPE threshold) {
+        cx_handle h = this->handle_.get();
+        const long long cap = max_message_bytes(vector_size);
+        cxx::Staged<const VarTYPE> d(h, this->stage_a_, data_vector, (size_t)(data_vector ? vector_size : 0), true, false);
+        cxx::Staged<VarTYPE> u(h, this->stage_b_, update_vector, (size_t)(update_vector ? vector_size : 0), true, true);
+        const bool host_out = !cx_pointer_on_device(output);
+        void* d_out = host_out ? this->stage_msg_.reserve((size_t)cap) : output;
+        const int bytes = compress_device(d_out, cap, data_vector ? d.get() : nullptr,
+                                          update_vector ? u.get() : nullptr, vector_size, nullptr, threshold, nullptr,
+                                          true);
+        if (host_out) cxx::check(cx_copy(h, output, d_out, (size_t)bytes));
+        u.flush();
+        cxx::check(cx_synchronize(h));
+        return bytes;
+    }
+
+    // a host-resident message is staged whole: its length follows from c and, behind the values, runs
+    const void* stage_message(const void* msg) {
+        if (cx_pointer_on_device(msg)) return msg;
+        const char* p = static_cast<const char*>(msg);
+        int c = 0, runs = 0;
+        std::memcpy(&c, p + 4, 4);
+        if (c < 0) c = 0;
+        std::memcpy(&runs, p + 8 + (size_t)c * sizeof(VarTYPE), 4);
+        if (runs < 0) runs = 0;
+        const size_t bytes = 16 + (size_t)c * sizeof(VarTYPE) + 4 * (size_t)runs;
+        void* d = this->stage_msg_.reserve(bytes);
+        cxx::check(cx_copy(this->handle_.get(), d, msg, bytes));
+        return d;
+    }
+
+    virtual int decompression_strategy(VarTYPE* output, int output_size, const void* input) {
+        cx_handle h = this->handle_.get();
+        const void* d_in = stage_message(input);
+        // only the message's n elements are written: a host vector is staged in and out
+        cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
+        const int n = decompress_device(o.get(), output_size, d_in, true);
+        o.flush();
+        cxx::check(cx_synchronize(h));
+        return n;
+    }
+    virtual void add_strategy(VarTYPE* output, int output_size, const void* sourceBuffer) {
+        cx_handle h = this->handle_.get();
+        const void* d_in = stage_message(sourceBuffer);
+        cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
+        add_device(o.get(), output_size, d_in);
         o.flush();
         cxx::check(cx_synchronize(h));
     }

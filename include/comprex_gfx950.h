@@ -152,6 +152,22 @@ int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_c
                         const void* data, void* update, int n, float topK,
                         void* d_thr_out, int* d_size_prefix, int* h_bytes);
 
+/* CompressorRLE<T> (src/compressor.hxx:158-532), the run-length codec: message
+ * int32 n | int32 c | c values | int32 runs | int32 signum | runs x int32 run lengths, an element
+ * is sent when |x| >= threshold.  cx_rle_compress = compression_strategy (:167-390) in its three
+ * modes (arguments as cx_ip_compress), with the sent values stored densely: the reference's
+ * encoder indexes them by vector position (:238,277,316) and only produces a decodable message
+ * when every element is sent.  cx_rle_decompress = decompression_strategy (:393-470): writes
+ * the message's n elements (nothing beyond), *h_n receives n, which is what the reference
+ * returns; CX_ERR_MSG_TOO_LARGE when n > out_n.  cx_rle_add = add_strategy (:473-530).
+ * The two decoders read the message's header on the host (they wait for the stream). */
+int cx_rle_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity,
+                    const void* data, void* update, int n,
+                    const void* thr_host, const void* d_thr,
+                    int* d_size_prefix, int* h_bytes);
+int cx_rle_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_n);
+int cx_rle_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg);
+
 /* CompressorIndexPairs<T>::decompression_strategy (src/compressor.hxx:613-638): zero
  * all out_n elements, then out[index] = value.  A message whose n exceeds out_n leaves
  * `out` zeroed and records CX_ERR_MSG_TOO_LARGE.  h_bytes as above (bytes consumed). */
@@ -220,6 +236,8 @@ void ThresholdTopK_del(void* self);
 float ThresholdTopK_getThreshold(void* self);
 void* CompressorNone_new(void);
 void CompressorNone_del(void* self);
+void* CompressorRLE_new(void);
+void CompressorRLE_del(void* self);
 void* CompressorIndexPairs_new(void);
 void CompressorIndexPairs_del(void* self);
 /* src/allreduce_C.cpp:26-122, the three compressed schedules.  One object per simulated rank, driven

@@ -12,6 +12,8 @@
  *   src/threshold.hxx:19-50     ThresholdFunction::apply / apply_split
  *   src/compressor.hxx:24-76    Compressor wrappers (size check)
  *   src/compressor.hxx:538-661  CompressorIndexPairs (compress / decompress / add)
+ *   src/compressor.hxx:158-532  CompressorRLE (decoder and adder as they are; the encoder with its
+ *                               value-index bug corrected, see cxo_rle_compress)
  *   src/comprEx.tpp:121-246     residual maintenance, writeRemote*, flushRests, readRemote*
  *
  * Every function is pinned (tests/test_oracle_*.py) against: the compiled
@@ -94,6 +96,13 @@ int cxo_sample_count(int n, int subsamples);
     /* compressor.hxx:640-658 add_strategy: out[idx] += val in message order.  Returns 0,     \
      * or -1 when the message's vector size exceeds out_n (nothing modified). */              \
     int cxo_ip_add_##SFX(T* out, int out_n, const void* in);                                  \
+    /* compressor.hxx:158-532 CompressorRLE: int32 n, int32 c, c values, int32 runs, int32 signum,  \
+     * run lengths; an element is sent when |x| >= thr.  The encoder stores the sent values      \
+     * densely, where the reference's encoder indexes them by vector position (its bug at        \
+     * :238,277,316); decoder and adder as the reference's.  -1: no input vector / n > out_n. */ \
+    int cxo_rle_compress_##SFX(void* out, const T* data, T* update, int n, T thr);               \
+    int cxo_rle_decompress_##SFX(T* out, int out_n, const void* in);                             \
+    int cxo_rle_add_##SFX(T* out, int out_n, const void* in);                                    \
     /* comprEx.tpp:159-169 addRests: data[i] += rests[i]. */                                  \
     void cxo_add_rests_##SFX(T* data, const T* rests, int n);                                 \
     /* comprEx.tpp:176-191 writeRemote: prepare_with + compress_add_update into               \

@@ -169,6 +169,39 @@ class Oracle:
         if r < 0:
             raise RuntimeError("Decompression vector size is bigger than output buffer!")
 
+    # ---- run-length codec ---------------------------------------------
+    @staticmethod
+    def rle_capacity(n, dtype):
+        return 16 + n * np.dtype(dtype).itemsize + 4 * (n + 1)
+
+    def rle_compress(self, data, update, thr, out=None):
+        """data and/or update (update is modified in place).  Returns the message bytes.  With
+        ref=True this is the reference's encoder, which is only sound when every element is sent."""
+        ref_arr = data if data is not None else update
+        s = self._sfx(ref_arr)
+        n = ref_arr.size
+        if out is None:
+            out = np.zeros(self.rle_capacity(n, ref_arr.dtype) + 8 * n, dtype=np.uint8)
+        nbytes = self._f("rle_compress_" + s, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, _CT[s])(
+            _ptr(out), _ptr(data), _ptr(update), n, thr)
+        return out[:nbytes]
+
+    def rle_decompress(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("rle_decompress_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(
+            _ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+        return r
+
+    def rle_add(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("rle_add_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(_ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+
     # ---- channel level (restatement only) ----------------------------
     def add_rests(self, data, rests):
         assert not self.ref

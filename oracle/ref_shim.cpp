@@ -93,6 +93,30 @@ int cxr_calc_subsamples(float topK, int default_subsamples, float subsample_fact
         return 0;                                                                                 \
     }
 
+/* the reference's run-length codec: its decoder and adder on any message, its encoder only
+ * where it is sound (every element sent) */
+#define CXR_DEFINE_RLE(SFX, T)                                                                    \
+    int cxr_rle_compress_##SFX(void* out, const T* data, T* update, int n, T thr) {               \
+        CompressorRLE<T> c;                                                                       \
+        if (data && update) return c.compress_add_update(out, update, n, data, n, thr);           \
+        if (update) return c.compress_update(out, update, n, thr);                                \
+        return c.compress(out, data, n, thr);                                                     \
+    }                                                                                             \
+    int cxr_rle_decompress_##SFX(T* out, int out_n, const void* in) {                             \
+        CompressorRLE<T> c;                                                                       \
+        try { return c.decompress(out, out_n, in); }                                              \
+        catch (const std::runtime_error&) { return -1; }                                          \
+    }                                                                                             \
+    int cxr_rle_add_##SFX(T* out, int out_n, const void* in) {                                    \
+        CompressorRLE<T> c;                                                                       \
+        try { c.add(out, out_n, in); }                                                            \
+        catch (const std::runtime_error&) { return -1; }                                          \
+        return 0;                                                                                 \
+    }
+CXR_DEFINE_RLE(f32, float)
+CXR_DEFINE_RLE(f64, double)
+CXR_DEFINE_RLE(i32, int)
+
 CXR_DEFINE(f32, float)
 CXR_DEFINE(f64, double)
 CXR_DEFINE(i32, int)

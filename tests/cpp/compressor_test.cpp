@@ -1,6 +1,6 @@
-// Mirrors the reference's test/compressor.cpp for CompressorIndexPairs (the run-length codec is
-// not provided): compress(threshold 0) then decompress reproduces the input; plus add(), the
-// fused compress_add_update and the error paths of src/compressor.hxx:44-51,620-624,645-647.
+// Mirrors the reference's test/compressor.cpp for CompressorRLE and CompressorIndexPairs:
+// compress(threshold 0) then decompress reproduces the input; plus add(), the fused
+// compress_add_update and the error paths of src/compressor.hxx:44-51,620-624,645-647.
 #include <compressor.hxx>
 
 #include <cstdlib>
@@ -18,6 +18,35 @@ template <typename data_t> int run(const char* name) {
         if (e != 0) ++nelem;
     char buffer[16 * size];
 
+    {  // run-length codec: round trip at threshold 0 (test/compressor.cpp:43-68), then a real threshold
+        int errors = 0;
+        std::vector<data_t> myValues(values);
+        CompressorRLE<data_t> compressor;
+        std::cout << "Test CompressorRLE class (" << name << ")." << std::endl;
+        const int bytes = compressor.compress(reinterpret_cast<void*>(buffer), myValues.data(), (int)myValues.size(), 0);
+        if (bytes != 16 + size * (int)sizeof(data_t) + 4) ++errors;  // every element sent: one run
+        std::vector<data_t> out_vec(size, (data_t)7);
+        if (compressor.decompress(out_vec.data(), (int)out_vec.size(), reinterpret_cast<void*>(buffer)) != size) ++errors;
+        for (int i = 0; i < size; ++i)
+            if (out_vec[i] != values[i]) ++errors;
+        // |x| >= 50 sent, residual keeps the rest; decompress + residual == input
+        std::vector<data_t> rest(values);
+        compressor.compress_update(reinterpret_cast<void*>(buffer), rest.data(), size, (data_t)50);
+        std::vector<data_t> sent(size + 3, (data_t)7);
+        compressor.decompress(sent.data(), size + 3, reinterpret_cast<void*>(buffer));
+        for (int i = 0; i < size; ++i) {
+            const bool big = std::abs(values[i]) >= (data_t)50;
+            if (sent[i] != (big ? values[i] : (data_t)0) || rest[i] != (big ? (data_t)0 : values[i])) ++errors;
+        }
+        for (int i = size; i < size + 3; ++i)
+            if (sent[i] != (data_t)7) ++errors;  // nothing beyond the message's vector is written
+        std::vector<data_t> acc(size, (data_t)1);
+        compressor.add(acc.data(), size, reinterpret_cast<void*>(buffer));
+        for (int i = 0; i < size; ++i)
+            if (acc[i] != (data_t)(1 + sent[i])) ++errors;
+        try { compressor.decompress(sent.data(), size - 1, reinterpret_cast<void*>(buffer)); ++errors; } catch (const std::runtime_error&) {}
+        failed += print_pass(errors);
+    }
     {  // round trip  (test/compressor.cpp:70-94)
         int errors = 0;
         std::vector<data_t> myValues(values);

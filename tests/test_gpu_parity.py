@@ -585,3 +585,107 @@ def test_small_golden_fixtures(dev):
         o = _gpu(grads[0])
         dev.add(o, m0)
         assert o.cpu().numpy().tobytes() == z[key + "_add0"].tobytes()
+
+
+# --------------------------------------------------------------------------- run-length codec
+def _rle_buf(n, dtype, extra=0):
+    return torch.zeros(16 + n * np.dtype(dtype).itemsize + 4 * (n + 1) + extra, dtype=torch.uint8, device="cuda")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mode", ["fused", "update", "data"])
+def test_rle_compress_matches_oracle(dev, oracle, dtype, mode):
+    """CompressorRLE: values + run lengths, |x| >= threshold, byte for byte as the checker, whose
+    encoder is pinned through the reference's own decoder."""
+    rng = np.random.default_rng(51)
+    for n in [0, 1, 2, 63, 64, 65, 1000, 4097, 100_003, 1_000_001]:
+        for q in [0.0, 0.5, 0.99, 0.9999, 1.5]:
+            say("rle compress", dtype.__name__, mode, n, q)
+            d = _rand(rng, n, dtype)
+            u = _rand(rng, n, dtype, 0.5)
+            ref = d if mode == "data" else (u if mode == "update" else (u + d).astype(dtype))
+            thr = dtype(0) if n == 0 or q == 0 else dtype(np.quantile(np.abs(ref), min(q, 1.0)) * (2 if q > 1 else 1))
+            dd = d.copy() if mode != "update" else None
+            uu = u.copy() if mode != "data" else None
+            if n == 0:
+                want = oracle.rle_compress(np.zeros(0, dtype), None, thr)
+            else:
+                want = oracle.rle_compress(dd, uu, thr)
+            gd = _gpu(d) if mode != "update" else None
+            gu = _gpu(u) if mode != "data" else None
+            if n == 0:
+                gd, gu = torch.zeros(0, dtype=NP2T[dtype], device="cuda"), None
+            buf = _rle_buf(n, dtype)
+            prefix = torch.zeros(1, dtype=torch.int32, device="cuda")
+            nbytes = dev.rle_compress(buf, gd, gu, thr=thr, size_prefix=prefix)
+            assert nbytes == want.size == int(prefix.item()), (n, q, nbytes, want.size)
+            assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes(), (n, q)
+            if gu is not None and n > 0:
+                assert gu.cpu().numpy().tobytes() == uu.tobytes()
+            if gd is not None and n > 0:
+                assert gd.cpu().numpy().tobytes() == d.tobytes()
+
+
+def test_rle_runs_of_every_shape_and_threshold_on_the_device(dev, oracle):
+    rng = np.random.default_rng(52)
+    n = 300_000
+    shapes = {
+        "alternating": np.where(np.arange(n) % 2 == 0, 5.0, 0.0),
+        "starts_unsent": np.where(np.arange(n) % 2 == 1, 5.0, 0.0),
+        "long_runs": np.where((np.arange(n) // 10_000) % 2 == 0, 3.0, 0.25),
+        "one_sent_at_the_end": np.where(np.arange(n) == n - 1, 9.0, 0.0),
+        "one_unsent_in_the_middle": np.where(np.arange(n) == n // 2, 0.0, 9.0),
+        "random_blocks": np.repeat(rng.random(n // 100) < 0.3, 100) * 4.0,
+        "equal_to_threshold": np.where(rng.random(n) < 0.1, 1.0, 0.5),  # |x| == thr is sent
+    }
+    d_thr = torch.tensor([1.0], device="cuda")
+    for name, v in shapes.items():
+        v = (v * np.where(rng.random(n) < 0.5, -1, 1)).astype(np.float32)
+        say("rle shape", name)
+        want = oracle.rle_compress(v, None, np.float32(1.0))
+        buf = _rle_buf(n, np.float32)
+        nbytes = dev.rle_compress(buf, _gpu(v), None, d_thr=d_thr)  # threshold read on the device
+        assert nbytes == want.size and buf[:nbytes].cpu().numpy().tobytes() == want.tobytes(), name
+        out = torch.full((n + 7,), 3.0, device="cuda")
+        assert dev.rle_decompress(out, buf) == n
+        assert out[:n].cpu().numpy().tobytes() == np.where(np.abs(v) >= 1, v, 0).astype(np.float32).tobytes(), name
+        assert bool((out[n:] == 3.0).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rle_decompress_add_match_oracle_and_errors(dev, oracle, dtype):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rng = np.random.default_rng(53)
+    for n in [1, 5, 1000, 70_001, 1_000_003]:
+        for q in [0.0, 0.9, 0.999]:
+            say("rle decode", dtype.__name__, n, q)
+            v = _rand(rng, n, dtype)
+            thr = dtype(0) if q == 0 else dtype(np.quantile(np.abs(v), q))
+            msg = oracle.rle_compress(v, None, thr)
+            gmsg = _gpu(msg)
+            base = _rand(rng, n + 9, dtype)
+            o = base.copy()
+            assert oracle.rle_decompress(msg, o) == n
+            g = _gpu(base)
+            assert dev.rle_decompress(g, gmsg) == n
+            assert g.cpu().numpy().tobytes() == o.tobytes()
+            o = base.copy()
+            oracle.rle_add(msg, o)
+            g = _gpu(base)
+            dev.rle_add(g, gmsg)
+            dev.synchronize()
+            assert g.cpu().numpy().tobytes() == o.tobytes()
+    with pytest.raises(ComprexError) as e:
+        dev.rle_decompress(torch.zeros(n - 1, dtype=NP2T[dtype], device="cuda"), gmsg)
+    assert e.value.code == _lib.CX_ERR_MSG_TOO_LARGE
+    with pytest.raises(ComprexError) as e:
+        dev.rle_add(torch.zeros(n - 1, dtype=NP2T[dtype], device="cuda"), gmsg)
+    assert e.value.code == _lib.CX_ERR_MSG_TOO_LARGE
+    # message buffer too small: reported, nothing written past the buffer
+    small = torch.zeros(64, dtype=torch.uint8, device="cuda")
+    guard = small.clone()
+    with pytest.raises(ComprexError) as e:
+        dev.rle_compress(small[:40], _gpu(v), None, thr=dtype(0))
+    assert e.value.code == _lib.CX_ERR_CAPACITY
+    assert torch.equal(small[40:], guard[40:])

@@ -305,3 +305,79 @@ def test_exact_mode_survivor_count(oracle):
     buf, thr = oracle.write_remote(r, g, np.float32(0.01), default_subsamples=1 << 17)
     k = parse_message(buf, np.float32)[1]
     assert k == oracle.topk_pos(n, np.float32(0.01)) == 655
+
+
+# --------------------------------------------------------------------------- run-length codec
+def _rle_parts(msg, dtype):
+    n, c = msg[:8].view(np.int32)
+    item = np.dtype(dtype).itemsize
+    vals = msg[8:8 + c * item].view(dtype)
+    runs, signum = msg[8 + c * item:16 + c * item].view(np.int32)
+    lens = msg[16 + c * item:16 + c * item + 4 * runs].view(np.int32)
+    assert msg.size == 16 + c * item + 4 * runs
+    return int(n), vals, int(signum), lens
+
+
+def test_rle_known_answers_by_hand(oracle):
+    """Small messages written out by hand from the layout the reference's decoder reads
+    (src/compressor.hxx:415-470): n, c, values, runs, signum, alternating run lengths."""
+    v = np.array([5, 0, 0, -7, 8, 0], np.int32)
+    n, vals, signum, lens = _rle_parts(oracle.rle_compress(v, None, np.int32(1)), np.int32)
+    assert (n, vals.tolist(), signum, lens.tolist()) == (6, [5, -7, 8], 1, [1, 2, 2, 1])
+    v = np.array([0, 0, 3, 0, 4, 4], np.int32)
+    n, vals, signum, lens = _rle_parts(oracle.rle_compress(v, None, np.int32(3)), np.int32)
+    assert (vals.tolist(), signum, lens.tolist()) == ([3, 4, 4], 0, [2, 1, 1, 2])
+    # |x| >= threshold: an element equal to the threshold is sent (IndexPairs would keep it)
+    n, vals, signum, lens = _rle_parts(oracle.rle_compress(v, None, np.int32(4)), np.int32)
+    assert (vals.tolist(), signum, lens.tolist()) == ([4, 4], 0, [4, 2])
+    # nothing sent: one "not sent" run over the whole vector
+    n, vals, signum, lens = _rle_parts(oracle.rle_compress(v, None, np.int32(9)), np.int32)
+    assert (vals.size, signum, lens.tolist()) == (0, 0, [6])
+    # fused mode: update += data, sent entries cleared
+    u, d = np.array([1, 1, 1, 1], np.float32), np.array([0, 2, -3, 0], np.float32)
+    n, vals, signum, lens = _rle_parts(oracle.rle_compress(d, u, np.float32(2.5)), np.float32)
+    assert (vals.tolist(), signum, lens.tolist()) == ([3.0], 0, [1, 1, 2]) and u.tolist() == [1, 0, -2, 1]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rle_encoder_equals_reference_where_the_reference_is_sound(oracle, refimpl, dtype):
+    """The reference's encoder indexes the sent values by vector position; with every element
+    sent (threshold 0: its own round-trip test, test/compressor.cpp:74-82) position and count
+    coincide and its output is well formed: same bytes in all three modes."""
+    rng = np.random.default_rng(5)
+    for n in [1, 2, 17, 1000]:
+        v = (rng.standard_normal(n) * 9).astype(dtype)
+        a = (rng.standard_normal(n) * 3).astype(dtype)
+        for mode in ("data", "update", "fused"):
+            outs = []
+            for impl in (oracle, refimpl):
+                d = v.copy() if mode != "update" else None
+                u = a.copy() if mode != "data" else None
+                outs.append((impl.rle_compress(d, u, dtype(0)).tobytes(), None if u is None else u.tobytes()))
+            assert outs[0] == outs[1], (n, mode)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rle_messages_decode_with_the_reference_decoder(oracle, refimpl, dtype):
+    """Messages of the corrected encoder through the reference's own decoder and adder give the
+    thresholded vector; the restated decoder and adder agree with the reference's byte for byte."""
+    rng = np.random.default_rng(6)
+    for n in [1, 2, 3, 64, 1000, 4097]:
+        for q in [0.0, 0.3, 0.9, 0.99, 1.1]:
+            v = (rng.standard_normal(n) * 50).astype(dtype)
+            thr = dtype(np.quantile(np.abs(v), min(q, 1.0)) + (1 if q > 1 else 0))
+            msg = oracle.rle_compress(v, None, thr)
+            want = np.where(np.abs(v) >= thr, v, 0).astype(dtype)
+            nn, vals, signum, lens = _rle_parts(msg, dtype)
+            assert nn == n and lens.sum() == n and (lens > 0).all()
+            assert vals.tobytes() == v[np.abs(v) >= thr].tobytes()
+            assert signum == int(np.abs(v[0]) >= thr)
+            for impl in (oracle, refimpl):
+                out = np.full(n + 5, 77, dtype)
+                assert impl.rle_decompress(msg, out) == n
+                assert out[:n].tobytes() == want.tobytes() and (out[n:] == 77).all()  # nothing beyond n is touched
+                acc = np.arange(n + 5).astype(dtype)
+                impl.rle_add(msg, acc)
+                assert acc[:n].tobytes() == (np.arange(n).astype(dtype) + want).astype(dtype).tobytes()
+                with pytest.raises(RuntimeError):
+                    impl.rle_decompress(msg, np.zeros(n - 1, dtype))
