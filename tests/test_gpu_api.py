@@ -26,14 +26,14 @@ def test_cpp_mirror_of_reference_tests(name):
     assert "+++ PASSED +++" in r.stdout and "--- FAILED ---" not in r.stdout
 
 
-def _pair(env, n, size_factor=3.0, topk=0.01, tag=1):
+def _pair(env, n, size_factor=3.0, topk=0.01, tag=1, compressor="CompressorIndexPairs"):
     from comprex_amd import pygpi
     objs = []
     for rank in range(2):
         env.set_rank(rank, 2)
         c = pygpi.Comprex(env, n, size_factor)
         c.setThreshold(pygpi.ThresholdTopK(topk))
-        c.setCompressor(pygpi.CompressorIndexPairs())
+        c.setCompressor(getattr(pygpi, compressor)())
         c.connectTo((rank + 1) % 2, (rank + 1) % 2, tag)
         objs.append(c)
     return objs
@@ -73,12 +73,14 @@ def test_reference_abi_matches_oracle(oracle, on_device):
     assert not tx.getRests().any()
 
 
-def test_reference_abi_conservation_and_errors():
-    """test/comprex.cpp's gold through the Python wrappers, plus the errors the reference throws."""
+@pytest.mark.parametrize("compressor", ["CompressorIndexPairs", "CompressorRLE", "CompressorNone"])
+def test_reference_abi_conservation_and_errors(compressor):
+    """test/comprex.cpp's gold through the Python wrappers with each codec, plus the errors the
+    reference throws."""
     from comprex_amd import pygpi
     n = 50
     env = pygpi.GaspiEnvironment()
-    tx, rx = _pair(env, n, topk=0.1)
+    tx, rx = _pair(env, n, topk=0.1, compressor=compressor)
     i = np.arange(n)
     values = (i * (1 - 2 * (i % 2))).astype(np.float32)
     result = np.zeros(n, np.float32)
