@@ -26,6 +26,22 @@ def test_cpp_mirror_of_reference_tests(name):
     assert "+++ PASSED +++" in r.stdout and "--- FAILED ---" not in r.stdout
 
 
+@pytest.mark.parametrize("name,passes", [("refsrc_threshold", 2), ("refsrc_compressor", 2)])
+def test_reference_own_test_sources_against_these_headers(name, passes):
+    """test/threshold.cpp and test/compressor.cpp of the reference, compiled UNCHANGED with this
+    repository's include/ in front of the reference's src/ (tests/cpp/Makefile, target refsrc) and
+    linked to the HIP library: the drop-in claim at the C++ source level.  The binaries exist where
+    the reference tree was present at build time."""
+    exe = os.path.join(BIN, name)
+    if not os.path.exists(exe):
+        pytest.skip("built only where the reference tree is present")
+    print("running", exe, file=sys.stderr, flush=True)
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    sys.stderr.write(r.stdout[-2000:] + r.stderr[-2000:])
+    assert r.returncode == 0
+    assert r.stdout.count("+++ PASSED +++") == passes and "--- FAILED ---" not in r.stdout
+
+
 def _pair(env, n, size_factor=3.0, topk=0.01, tag=1, compressor="CompressorIndexPairs"):
     from comprex_amd import pygpi
     objs = []
