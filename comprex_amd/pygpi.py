@@ -78,6 +78,17 @@ class Getable(object):
     def get(self):
         return self.obj
 
+    def _release(self, symbol):
+        """Calls the C destructor once; silent when the interpreter is already tearing the module down."""
+        obj = getattr(self, "obj", None)
+        if not obj:
+            return
+        self.obj = None
+        try:
+            getattr(libcomprex(), symbol)(obj)
+        except TypeError:  # module globals are gone at interpreter exit
+            pass
+
 
 class GaspiEnvironment(Getable):
     def __init__(self, segment_size=1 << 20):
@@ -85,9 +96,7 @@ class GaspiEnvironment(Getable):
         _raise_if_failed()
 
     def __del__(self):
-        if getattr(self, "obj", None):
-            libcomprex().GaspiEnvironment_del(self.obj)
-            self.obj = None
+        self._release("GaspiEnvironment_del")
 
     def get_rank(self):
         return libcomprex().GaspiEnvironment_get_rank(self.obj)
@@ -111,7 +120,7 @@ class GaspiEnvironment(Getable):
         libcomprex().GaspiEnvironment_flush(self.obj)
 
 
-class Comprex(object):
+class Comprex(Getable):
     def __init__(self, gaspi_env, size, size_factor=1.0):
         self.size = size
         self.env = gaspi_env  # keeps the channel registry alive
@@ -119,9 +128,7 @@ class Comprex(object):
         _raise_if_failed()
 
     def __del__(self):
-        if getattr(self, "obj", None) is not None:
-            libcomprex().Comprex_del(self.obj)
-            self.obj = None
+        self._release("Comprex_del")
 
     def setThreshold(self, threshold):
         libcomprex().Comprex_setThreshold(self.obj, threshold.get())
@@ -187,7 +194,7 @@ class ThresholdNone(Getable):
         self.obj = libcomprex().ThresholdNone_new()
 
     def __del__(self):
-        libcomprex().ThresholdNone_del(self.obj)
+        self._release("ThresholdNone_del")
 
 
 class ThresholdConst(Getable):
@@ -196,8 +203,7 @@ class ThresholdConst(Getable):
         _raise_if_failed()
 
     def __del__(self):
-        if self.obj:
-            libcomprex().ThresholdConst_del(self.obj)
+        self._release("ThresholdConst_del")
 
     def getThreshold(self):
         return libcomprex().ThresholdConst_getThreshold(self.obj)
@@ -209,8 +215,7 @@ class ThresholdTopK(Getable):
         _raise_if_failed()
 
     def __del__(self):
-        if self.obj:
-            libcomprex().ThresholdTopK_del(self.obj)
+        self._release("ThresholdTopK_del")
 
     def getThreshold(self):
         return libcomprex().ThresholdTopK_getThreshold(self.obj)
@@ -221,7 +226,7 @@ class CompressorNone(Getable):
         self.obj = libcomprex().CompressorNone_new()
 
     def __del__(self):
-        libcomprex().CompressorNone_del(self.obj)
+        self._release("CompressorNone_del")
 
 
 class CompressorRLE(Getable):
@@ -229,7 +234,7 @@ class CompressorRLE(Getable):
         self.obj = libcomprex().CompressorRLE_new()
 
     def __del__(self):
-        libcomprex().CompressorRLE_del(self.obj)
+        self._release("CompressorRLE_del")
 
 
 class CompressorIndexPairs(Getable):
@@ -237,7 +242,7 @@ class CompressorIndexPairs(Getable):
         self.obj = libcomprex().CompressorIndexPairs_new()
 
     def __del__(self):
-        libcomprex().CompressorIndexPairs_del(self.obj)
+        self._release("CompressorIndexPairs_del")
 
 
 ###########################
@@ -253,9 +258,7 @@ class _ComprexAllreduce(Getable):
         _raise_if_failed()
 
     def __del__(self):
-        if getattr(self, "obj", None):
-            getattr(libcomprex(), self._family + "_del")(self.obj)
-            self.obj = None
+        self._release(self._family + "_del")
 
     def apply(self, vector):
         """In place on `vector` (float32 numpy array or CUDA tensor); returns it."""
