@@ -107,7 +107,8 @@ struct cx_handle_s {
     unsigned* rle_scan = nullptr;      // run-length codec: per-block counts / prefix sums over the runs
     size_t rle_scan_bytes = 0;
     cx::DeviceStatus* d_status = nullptr;
-    void* d_thr = nullptr;             // 8-byte threshold slot
+    void* d_thr = nullptr;             // 256 bytes: threshold slot at 0, sampled lower bound at 64,
+                                       // small result words at 128, a codec's derived threshold at 192
     int* h_pinned = nullptr;           // 64-byte pinned read-back area
 
     // optional timing of the streaming pass: HIP events recorded around stage_kernel
