@@ -23,7 +23,6 @@ namespace cx {
 namespace {
 
 constexpr int kBlock = 256;
-constexpr int kSmallSelect = 1 << 18;  // sample sets up to this size take the two-launch path
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -215,15 +214,29 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
     }
 }
 
-// ---- small sample sets: two launches ---------------------------------------------------
-// First launch: one thread per sample gathers its key, stores it to `keys` and counts the top
-// digit.  Second launch, one block: picks the top digit and finishes the remaining digits alone;
-// when the keys sharing the picked top digit fit in LDS they are collected there in one scan of
-// `keys` and the other passes never leave LDS, else every pass scans `keys` again.
+// ---- up to 2^18 keys: two launches --------------------------------------------------------
+// First launch: every block gathers KPT keys per thread, stores them to `keys` and counts their
+// top digit.  Second launch, one block: picks the top digit and finishes the remaining digits
+// alone, in LDS as soon as the keys still in play fit there.
+//
+// One block has the instruction throughput and the memory bandwidth of one compute unit
+// (measured: about 50 GB/s, 7 us per 100 000 four-byte keys), so the second launch must not read
+// every key.  When the wanted key is near the top, each block of the first launch also passes on a
+// SHORT LIST: its keys from the top digit of its own short_k-th largest key upwards (all its keys
+// when it has fewer), and the largest such digit over all blocks is recorded.  If the digit the
+// second launch picks is not below that, every key carrying it is in the short list and the
+// full key array is not needed; otherwise (large keys clustered in a few blocks, ties) the
+// second launch reads the key array, as it does when no short list was made.
 constexpr int kFinishBlock = 1024;
-constexpr int kShortListBytes = 32768;  // LDS list of the second launch, and the first launch's short list
+constexpr int kListBytes = 32768;           // LDS list of the second launch
+constexpr int kShortGlobalKeys = 1 << 16;   // capacity of the short list in device memory
+// Largest key count of this path.  Four keys per thread and 2^20 keys were measured too: no faster
+// than three histogram passes over the vector (63 vs 68 us at 2^20 keys), and the second
+// launch's worst case (no usable short list: it reads every key, up to three times) grows with
+// the key count.
+constexpr int kSmallSelect = 1 << 18;
 
-template <typename T, int SMODE, bool HAS_ADD>
+template <typename T, int SMODE, bool HAS_ADD, int KPT>
 __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                               const int* __restrict__ idx, int m, int n, float stepsize,
                                                               typename Elem<T>::key_t* __restrict__ keys,
@@ -232,28 +245,30 @@ __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __r
                                                               unsigned short_cap) {
     using key_t = typename Elem<T>::key_t;
     constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
+    constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit, s_base, s_wave[kFinishBlock / 64];
     __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
-    key_t mine = 0;       // with short_k > 0 the grid covers m: one key per thread
-    bool have = false;
     // large blocks: every block ends with one global atomic per digit it has seen, and those
     // queue up per address
     for (int b = threadIdx.x; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
     __syncthreads();
-    const int stride = gridDim.x * kFinishBlock;
-    // whole wavefronts stay in the loop together (hist_add is a cross-lane operation)
-    for (int i0 = blockIdx.x * kFinishBlock; i0 < m; i0 += stride) {
-        const int i = i0 + threadIdx.x;
+    key_t mine[KPT];
+    bool have[KPT];
+    // the grid covers m; whole wavefronts take every step together (hist_add is a cross-lane operation)
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+        const long long i = ((long long)blockIdx.x * KPT + q) * kFinishBlock + threadIdx.x;
         key_t k = 0;
-        if (i < m) {
+        have[q] = i < m;
+        if (have[q]) {
             long long p;
             bool ok = true;
             if (SMODE == 0) {
                 p = i;
             } else if (SMODE == 1) {
-                p = (long long)(int)__fmul_rn((float)i, stepsize);  // (int)(i * stepsize), product in fp32
-                if (p > (long long)n - 1) p = (long long)n - 1;     // the reference would read out of bounds
+                p = (long long)(int)__fmul_rn((float)(int)i, stepsize);  // (int)(i * stepsize), product in fp32
+                if (p > (long long)n - 1) p = (long long)n - 1;          // the reference would read out of bounds
                 if (p < 0) p = 0;
             } else {
                 p = idx[i];
@@ -264,28 +279,31 @@ __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __r
             if (HAS_ADD) v = (T)(v + add[p]);
             k = ok ? key_of(v) : (key_t)0;
             keys[i] = k;
-            mine = k;
-            have = true;
         }
-        hist_add(lds_hist, i < m, (unsigned)(k >> shift0) & ((1u << kRadixBits) - 1u));
+        mine[q] = k;
+        hist_add(lds_hist, have[q], (unsigned)(k >> shift0) & kDigitMask);
     }
     merge_hist<kFinishBlock>(lds_hist, st);
     if (short_k <= 0) return;
 
-    // Short list: the single-block second launch is bound by how many keys it must read, and
-    // the key it looks for is near the top.  Each block passes on only its keys from the top
-    // digit of its own short_k-th largest key upwards (all its keys when it has fewer), and the
-    // largest such digit over all blocks is recorded.  If the digit the second launch picks is
-    // not below that, every key carrying it is in the short list, and the full key array is not
-    // needed.
     unsigned digit;
     unsigned long long above;
     block_pick<kFinishBlock>(lds_hist, (unsigned long long)(short_k - 1), s_sum, &s_digit, &s_above, digit, above);
-    const unsigned my_digit = (unsigned)(mine >> shift0) & ((1u << kRadixBits) - 1u);
-    const bool out = have && my_digit >= digit;
+    unsigned outs = 0, cnt = 0;  // bit q: key q goes to the short list
+#pragma unroll
+    for (int q = 0; q < KPT; ++q) {
+        const bool out = have[q] && ((unsigned)(mine[q] >> shift0) & kDigitMask) >= digit;
+        outs |= (out ? 1u : 0u) << q;
+        cnt += out ? 1u : 0u;
+    }
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned long long votes = __ballot(out);
-    if (lane == 0) s_wave[wave] = (unsigned)__popcll(votes);
+    unsigned incl = cnt;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned up = __shfl_up(incl, o, 64);
+        if (lane >= o) incl += up;
+    }
+    if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
     if (threadIdx.x == 0) {
         unsigned total = 0;
@@ -294,9 +312,56 @@ __global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __r
         atomicMax(&st->short_digit, digit);
     }
     __syncthreads();
-    unsigned at = s_base + (unsigned)__popcll(votes & (lane == 0 ? 0ull : (~0ull >> (64 - lane))));
+    unsigned at = s_base + incl - cnt;
     for (int w = 0; w < wave; ++w) at += s_wave[w];
-    if (out && at < short_cap) short_keys[at] = mine;  // an overflowing list is seen from its count
+#pragma unroll
+    for (int q = 0; q < KPT; ++q)
+        if ((outs >> q) & 1u) {
+            if (at < short_cap) short_keys[at] = mine[q];  // an overflowing list is seen from its count
+            ++at;
+        }
+}
+
+// One block walks `count` keys that start on a 16-byte boundary and hands every key that still
+// matches the fixed digits to `hit`.  Written for one compute unit: sixteen 16-byte loads per lane
+// are in flight per round (a round trip to memory per round, not per key), and the test costs two
+// instructions per key.
+template <typename KEY, typename HIT>
+__device__ __forceinline__ void scan_matching(const KEY* __restrict__ src, unsigned count, KEY prefix, KEY mask,
+                                              HIT hit) {
+    constexpr int KV = 16 / (int)sizeof(KEY);  // keys per 16-byte load
+    constexpr int kLoads = 16;
+    const int t = threadIdx.x;
+    const Pack<KEY, KV>* kv = reinterpret_cast<const Pack<KEY, KV>*>(src);
+    const int nfull = (int)(count / KV);
+    for (int v0 = 0; v0 < nfull; v0 += kFinishBlock * kLoads) {
+        Pack<KEY, KV> kk[kLoads];
+#pragma unroll
+        for (int q = 0; q < kLoads; ++q) {
+            const int v = v0 + q * kFinishBlock + t;
+            if (v < nfull) {
+                kk[q] = kv[v];
+            } else {
+#pragma unroll
+                for (int c = 0; c < KV; ++c) kk[q].x[c] = ~prefix;  // never matches
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < kLoads; ++q) {
+            bool any = false;
+#pragma unroll
+            for (int c = 0; c < KV; ++c) any |= (kk[q].x[c] & mask) == prefix;
+            if (any) {
+#pragma unroll
+                for (int c = 0; c < KV; ++c)
+                    if ((kk[q].x[c] & mask) == prefix) hit(kk[q].x[c]);
+            }
+        }
+    }
+    for (unsigned i = (unsigned)nfull * KV + t; i < count; i += kFinishBlock) {  // fewer than KV keys
+        const KEY k1 = src[i];
+        if ((k1 & mask) == prefix) hit(k1);
+    }
 }
 
 template <typename T>
@@ -304,11 +369,12 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
                                                                      int m, SelectState* __restrict__ st,
                                                                      unsigned long long rank, int plus_one,
                                                                      T* __restrict__ thr_out, int short_on,
-                                                                     const typename Elem<T>::key_t* __restrict__ short_keys) {
+                                                                     const typename Elem<T>::key_t* __restrict__ short_keys,
+                                                                     unsigned short_cap) {
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
-    constexpr int kListKeys = kShortListBytes / (int)sizeof(key_t);
+    constexpr int kListKeys = kListBytes / (int)sizeof(key_t);
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ key_t s_list[kListKeys];
     __shared__ unsigned s_digit, s_fill;
@@ -329,7 +395,11 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         st->short_digit = 0u;
     }
     key_t prefix = 0, mask = 0;
-    unsigned listed = 0;  // keys in s_list (0 = scan `keys`)
+    // where the keys still in play are read from: the key array, the short list, or (listed) LDS
+    const key_t* src = keys;
+    unsigned src_n = (unsigned)m;
+    bool listed = false;
+    unsigned list_n = 0;
     for (int p = 0; p < kPasses; ++p) {
         int shift = kKeyBits - kRadixBits * (p + 1);
         int bits = kRadixBits;
@@ -342,15 +412,14 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
             __syncthreads();
             if (listed) {
-                for (unsigned i = t; i < listed; i += kFinishBlock) {
+                for (unsigned i = t; i < list_n; i += kFinishBlock) {
                     const key_t k1 = s_list[i];
                     if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 }
             } else {
-                for (int i = t; i < m; i += kFinishBlock) {
-                    const key_t k1 = keys[i];
-                    if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
-                }
+                scan_matching<key_t>(src, src_n, prefix, mask, [&](key_t k1) {
+                    atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
+                });
             }
             __syncthreads();
         }
@@ -361,60 +430,19 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         prefix |= (key_t)digit << shift;
         mask |= (key_t)((1ull << bits) - 1ull) << shift;
         rank -= above;
-        if (p == 0 && short_on && short_count <= (unsigned)kListKeys && digit >= short_digit) {
-            // the short list holds every key with the picked top digit: keep those
+        if (p == 0 && short_on && short_count <= short_cap && digit >= short_digit) {
+            src = short_keys;  // holds every key with the picked top digit
+            src_n = short_count;
+        }
+        if (!listed && p + 1 < kPasses && in_digit <= (unsigned)kListKeys) {
+            // collect the keys still in play; their order does not matter
             if (t == 0) s_fill = 0u;
             __syncthreads();
-            for (unsigned i = t; i < short_count; i += kFinishBlock) {
-                const key_t k1 = short_keys[i];
-                if ((k1 & mask) == prefix) s_list[atomicAdd(&s_fill, 1u)] = k1;
-            }
+            scan_matching<key_t>(src, src_n, prefix, mask, [&](key_t k1) { s_list[atomicAdd(&s_fill, 1u)] = k1; });
             __syncthreads();
-            listed = s_fill;
-        } else if (p == 0 && in_digit <= (unsigned)kListKeys) {
-            // collect the keys that carry the picked top digit; their order does not matter.
-            if (t == 0) s_fill = 0u;
-            __syncthreads();
-            // One block has the instruction throughput and the memory bandwidth of one compute unit
-            // (measured: about 50 GB/s, 7 us per 100 000 four-byte keys), so the scan is written
-            // for few instructions per key: a lane counts its hits in a 16-byte load, reserves room
-            // for them with one LDS atomic (only lanes with hits take part), and stores them.
-            constexpr int KV = 16 / (int)sizeof(key_t);  // keys per 16-byte load
-            constexpr int kLoads = 16;  // 16-byte loads in flight per lane: a round trip to memory per round
-            const Pack<key_t, KV>* kv = reinterpret_cast<const Pack<key_t, KV>*>(keys);
-            const int nfull = m / KV;
-            for (int v0 = 0; v0 < nfull; v0 += kFinishBlock * kLoads) {
-                Pack<key_t, KV> kk[kLoads];
-#pragma unroll
-                for (int q = 0; q < kLoads; ++q) {
-                    const int v = v0 + q * kFinishBlock + t;
-                    if (v < nfull) {
-                        kk[q] = kv[v];
-                    } else {
-#pragma unroll
-                        for (int c = 0; c < KV; ++c) kk[q].x[c] = ~prefix;  // never matches
-                    }
-                }
-#pragma unroll
-                for (int q = 0; q < kLoads; ++q) {
-                    unsigned hits = 0;
-#pragma unroll
-                    for (int c = 0; c < KV; ++c) hits += ((kk[q].x[c] & mask) == prefix) ? 1u : 0u;
-                    if (hits) {
-                        unsigned at = atomicAdd(&s_fill, hits);
-#pragma unroll
-                        for (int c = 0; c < KV; ++c)
-                            if ((kk[q].x[c] & mask) == prefix) s_list[at++] = kk[q].x[c];
-                    }
-                }
-            }
-            for (int i = nfull * KV + t; i < m; i += kFinishBlock) {  // fewer than KV keys
-                const key_t k1 = keys[i];
-                if ((k1 & mask) == prefix) s_list[atomicAdd(&s_fill, 1u)] = k1;
-            }
-            __syncthreads();
-            listed = s_fill;
-            }
+            list_n = s_fill;
+            listed = true;
+        }
         __syncthreads();
     }
     if (t == 0) {
@@ -570,42 +598,44 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
     using key_t = typename Elem<T>::key_t;
 
     if (m <= kSmallSelect) {
-        if ((size_t)m * sizeof(key_t) > h->sel_keys_bytes) {
+        // key array (2 MB), then the short list
+        const size_t want_bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
+        if (h->sel_keys_bytes < want_bytes) {
             CX_HIP(hipStreamSynchronize(h->stream));
             if (h->sel_keys) CX_HIP(hipFree(h->sel_keys));
             h->sel_keys = nullptr;
             h->sel_keys_bytes = 0;
-            size_t bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
-            CX_HIP(hipMalloc(&h->sel_keys, bytes + kShortListBytes));  // key array, then the short list
-            h->sel_keys_bytes = bytes;
+            CX_HIP(hipMalloc(&h->sel_keys, want_bytes + (size_t)kShortGlobalKeys * sizeof(unsigned long long)));
+            h->sel_keys_bytes = want_bytes;
         }
         key_t* keys = static_cast<key_t*>(h->sel_keys);
-        key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) +
-                                                     (size_t)kSmallSelect * sizeof(unsigned long long));
-        const int blocks = (m + kFinishBlock - 1) / kFinishBlock;
+        key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) + h->sel_keys_bytes);
+        constexpr int kpt = 1;  // keys per thread of the first launch
+        const int per_block = kFinishBlock * kpt;
+        const int blocks = (m + per_block - 1) / per_block;
         // short list: worth it when the wanted rank is near the top, so that a block's share of the
         // keys above it (plus 8 sigma) is a small part of the block, and the shares fit the list
-        const unsigned short_cap = (unsigned)(kShortListBytes / (int)sizeof(key_t));
+        const unsigned short_cap = (unsigned)kShortGlobalKeys;
         const double share = (double)(rank + 1) / (double)blocks;
         int short_k = (int)(share + 8.0 * std::sqrt(share) + 8.0);
-        if (!h->select_short_list || m < 8192 || short_k > kFinishBlock / 4 ||
-            (double)blocks * (short_k + 16) > (double)short_cap)
+        if (!h->select_short_list || m < 8192 || short_k > per_block / 4 ||
+            (double)blocks * (short_k + 16.0 * kpt) > (double)short_cap)
             short_k = 0;
-#define CX_FIRST(SM, HA)                                                                                              \
-    hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kFinishBlock), 0, h->stream, vec, add_vec, \
-                       d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
-        if (add_vec) {
-            if (sample_mode == kSampleFull) CX_FIRST(0, true);
-            else if (sample_mode == kSampleStrided) CX_FIRST(1, true);
-            else CX_FIRST(2, true);
-        } else {
-            if (sample_mode == kSampleFull) CX_FIRST(0, false);
-            else if (sample_mode == kSampleStrided) CX_FIRST(1, false);
-            else CX_FIRST(2, false);
-        }
+#define CX_FIRST(SM, HA, KPT)                                                                                           \
+    hipLaunchKernelGGL((select_first_kernel<T, SM, HA, KPT>), dim3(blocks), dim3(kFinishBlock), 0, h->stream, vec,      \
+                       add_vec, d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
+#define CX_FIRST_MODE(HA, KPT)                                   \
+    do {                                                         \
+        if (sample_mode == kSampleFull) CX_FIRST(0, HA, KPT);    \
+        else if (sample_mode == kSampleStrided) CX_FIRST(1, HA, KPT); \
+        else CX_FIRST(2, HA, KPT);                               \
+    } while (0)
+        if (add_vec) CX_FIRST_MODE(true, kpt);
+        else CX_FIRST_MODE(false, kpt);
+#undef CX_FIRST_MODE
 #undef CX_FIRST
         hipLaunchKernelGGL(select_finish_kernel<T>, dim3(1), dim3(kFinishBlock), 0, h->stream, keys, m, h->sel, rank,
-                           plus_one, d_thr_out, short_k > 0 ? 1 : 0, short_keys);
+                           plus_one, d_thr_out, short_k > 0 ? 1 : 0, short_keys, short_cap);
         CX_HIP(hipGetLastError());
         return CX_OK;
     }

@@ -349,7 +349,7 @@ def test_sampled_threshold_short_list_and_inputs_that_defeat_it(dev, oracle, dty
         for name, v, a in [("spread", spread, add), ("clustered", clustered, zero), ("equal", equal, zero)]:
             gv, ga = _gpu(v), _gpu(a)
             for m, topk in [(100_000, 0.01), (65_536, 0.0133), (8_192, 0.01), (200_000, 0.002), (100_000, 0.2),
-                            (262_144, 0.01), (5_000, 0.01)]:
+                            (262_144, 0.01), (5_000, 0.01), (262_145, 0.01), (700_001, 0.003)]:
                 idx = np.sort(rng.integers(0, n, m)).astype(np.int32)
                 want = oracle.topk_prepare_indexed(v, a, idx, np.float32(topk))
                 gi = _gpu(idx)
