@@ -137,25 +137,37 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
     unsigned total = 0;
     unsigned valid_mask[ITEMS];
 
+    // every load of the tile is issued before the first value is used: the cross-lane steps below
+    // would otherwise fence each pair of loads off from the next
+    Pack<T, VEC> uu[ITEMS], dd[ITEMS];
+    if (full) {
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-        const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
-        Pack<T, VEC> u, d;
-        unsigned valid = (1u << VEC) - 1u;
-        if (full) {
-            if (MODE != 2) u = load_pack<T, VEC>(update + e0, false);
-            if (MODE != 1) d = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
-        } else {
-            valid = 0;
+        for (int j = 0; j < ITEMS; ++j) {
+            const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
+            if (MODE != 2) uu[j] = load_pack<T, VEC>(update + e0, false);
+            if (MODE != 1) dd[j] = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
+            valid_mask[j] = (1u << VEC) - 1u;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
+            unsigned valid = 0;
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
                 const bool in = e0 + c < n;
-                u.x[c] = (MODE != 2 && in) ? update[e0 + c] : (T)0;
-                d.x[c] = (MODE != 1 && in) ? data[e0 + c] : (T)0;
+                uu[j].x[c] = (MODE != 2 && in) ? update[e0 + c] : (T)0;
+                dd[j].x[c] = (MODE != 1 && in) ? data[e0 + c] : (T)0;
                 valid |= (in ? 1u : 0u) << c;
             }
+            valid_mask[j] = valid;
         }
-        valid_mask[j] = valid;
+    }
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const Pack<T, VEC>& u = uu[j];
+        const Pack<T, VEC>& d = dd[j];
+        const unsigned valid = valid_mask[j];
         unsigned m = 0;
 #pragma unroll
         for (int c = 0; c < VEC; ++c) {
