@@ -148,6 +148,23 @@ def main():
              "hbm_peak_fraction_step": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS}
 
     if not args.no_extra:
+        # what plain streaming reaches on this GPU, for scale: a device copy (8n bytes) and an
+        # in-place add (12n bytes, the streaming kernel's own access pattern) through torch
+        probe = torch.empty_like(g)
+        for name, fn, nbytes in (("device_copy", lambda: probe.copy_(g), 8 * n),
+                                 ("inplace_add", lambda: probe.add_(g), 12 * n)):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            extra[name + "_GBps"] = nbytes / ((time.perf_counter() - t0) / 20) / 1e9
+        del probe
+        log("plain streaming on this GPU: copy %.0f GB/s, in-place add %.0f GB/s"
+            % (extra["device_copy_GBps"], extra["inplace_add_GBps"]))
+
         # exact top-k (radix select over all n) + compress, same vector
         rests.zero_()
         ds = W.C4["default_subsamples_exact"] if n == W.C4["n"] else 1 << 30
