@@ -267,8 +267,9 @@ int cx_set_option(cx_handle h, const char* key, int value) {
             h->profile_events = new hipEvent_t[2 * cx_handle_s::kProfileRing];
             for (int i = 0; i < 2 * cx_handle_s::kProfileRing; ++i) CX_HIP(hipEventCreate(&h->profile_events[i]));
         }
-        h->profile = value ? 1 : 0;
+        h->profile = value > 0 ? value : 0;
         h->profile_count = 0;
+        h->profile_tick = 0;
     } else if (!strcmp(key, "stage_alternate")) {
         h->stage_alternate = value ? 1 : 0;
     } else if (!strcmp(key, "select_bracket")) {

@@ -113,7 +113,8 @@ struct cx_handle_s {
 
     // optional timing of the streaming pass: HIP events recorded around stage_kernel
     static constexpr int kProfileRing = 1024;
-    int profile = 0;
+    int profile = 0;                   // N > 0: events around every N-th streaming launch
+    unsigned profile_tick = 0;
     int profile_count = 0;             // launches recorded since the last read
     hipEvent_t* profile_events = nullptr;  // 2 * kProfileRing events, created on first use
 

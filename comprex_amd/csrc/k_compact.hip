@@ -469,7 +469,8 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
 
     const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
     hipEvent_t* ev = nullptr;
-    if (h->profile && h->profile_events && h->profile_count < cx_handle_s::kProfileRing) {
+    if (h->profile && h->profile_events && h->profile_count < cx_handle_s::kProfileRing &&
+        (h->profile_tick++ % (unsigned)h->profile) == 0u) {  // every profile-th launch
         ev = h->profile_events + 2 * h->profile_count;
         h->profile_count += 1;
         CX_HIP(hipEventRecord(ev[0], h->stream));

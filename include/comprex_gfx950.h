@@ -88,9 +88,10 @@ int cx_set_option(cx_handle h, const char* key, int value);
  * (0 = threshold and compress as two steps, 1 = single pass, 2 = single pass abandoned). */
 int cx_get_option(cx_handle h, const char* key, int* value);
 
-/* No counterpart in the reference: a measurement aid.  After cx_set_option(h, "profile_stage", 1)
- * every cx_ip_compress records a HIP event before and after its streaming kernel, on the handle's
- * stream (at most 1024 launches between reads).  This call waits for the stream and returns the
+/* No counterpart in the reference: a measurement aid.  After cx_set_option(h, "profile_stage", N)
+ * every N-th cx_ip_compress records a HIP event before and after its streaming kernel, on the
+ * handle's stream (at most 1024 recorded launches between reads; the two events cost a few
+ * microseconds per recorded launch).  This call waits for the stream and returns the
  * elapsed milliseconds of those launches, oldest first, and forgets them. */
 int cx_profile_read(cx_handle h, float* ms_out, int max_out, int* n_out);
 
