@@ -40,12 +40,13 @@ constexpr int kBlock = CX_STAGE_BLOCK;  // threads of a streaming block: one til
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
 #ifndef CX_GATHER_UNROLL
-#define CX_GATHER_UNROLL 8
+#define CX_GATHER_UNROLL 4
 #endif
 #ifndef CX_GATHER_BLOCK
 #define CX_GATHER_BLOCK 256
 #endif
-constexpr int kGatherBlock = CX_GATHER_BLOCK;  // tiles per gather block
+constexpr int kGatherBlock = CX_GATHER_BLOCK;  // threads of a gather block
+constexpr int kGatherTiles = 64;                // tiles a gather block owns: one lane per tile in its scan
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -292,12 +293,13 @@ __global__ __launch_bounds__(kBlock) void redo_kernel(const T* __restrict__ data
     }
 }
 
-// Final offsets of the tiles and copy of the staged slots to their final place.  A block
-// owns kGatherBlock consecutive tiles: it adds up the per-block sums the streaming pass left
-// for the tiles before its own (16-byte loads), scans its own counts, and each wavefront moves the pairs of its 64 tiles
-// with lane-contiguous stores.  Deferred tiles are either processed here, by the wavefront
-// that owns them (inline_redo), or left to redo_kernel, which then needs offsets[].  The
-// block that owns the last tile writes the message header.
+// Final offsets of the tiles and copy of the staged slots to their final place.  A block owns
+// kGatherTiles (64) consecutive tiles: it adds up the per-block sums the streaming pass left for the
+// tiles before its own (16-byte loads), every wavefront scans the 64 counts (one lane per tile),
+// and all wavefronts together move the block's pairs with lane-contiguous stores, so that the
+// whole GPU takes part in what is a latency-bound copy.  Deferred tiles are either processed
+// here, shared out among the block's wavefronts (inline_redo), or left to redo_kernel, which then
+// needs offsets[].  The block that owns the last tile writes the message header.
 template <typename T, int MODE, int VEC, int ITEMS>
 __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     const T* __restrict__ data, T* __restrict__ update, long long n, const T* __restrict__ thr_ptr, T thr_val,
@@ -307,19 +309,17 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
     constexpr int kWaves = kGatherBlock / 64;
-    // pairs a lane moves per round: searches and loads of one round are independent, so a wavefront's
-    // whole share (about 64 tiles x 1 % x 1024 elements) is in flight at once
+    // pairs a lane moves per round: searches and loads of one round are independent
     constexpr int kCopyUnroll = CX_GATHER_UNROLL;
     __shared__ unsigned s_before[kWaves];
-    __shared__ unsigned s_wave_total[kWaves];
-    __shared__ unsigned s_off[kWaves][65];
+    __shared__ unsigned s_off[65];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
     unsigned before = 0;
     {
-        // stage blocks before this block's first tile: kGatherBlock / kWavesPerBlock per gather block
+        // stage blocks before this block's first tile: kGatherTiles / kWavesPerBlock per gather block
         const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
-        const unsigned nvec = blockIdx.x * (kGatherBlock / kWavesPerBlock / 4);
+        const unsigned nvec = blockIdx.x * (kGatherTiles / kWavesPerBlock / 4);
 #pragma unroll 8
         for (unsigned v = tid; v < nvec; v += kGatherBlock) {
             const uint4 c = b4[v];
@@ -330,7 +330,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
     if (lane == 0) s_before[wave] = before;
 
-    const unsigned first = blockIdx.x * kGatherBlock + wave * 64u;
+    // every wavefront scans the same 64 counts
+    const unsigned first = blockIdx.x * kGatherTiles;
     const unsigned tile = first + lane;  // tiles past the end count as empty
     const unsigned raw = tile < ntiles ? counts[tile] : 0u;
     const unsigned cnt = raw & ~kDeferred;
@@ -340,47 +341,44 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
         const unsigned up = __shfl_up(incl, o, 64);
         if (lane >= o) incl += up;
     }
-    unsigned* so = s_off[wave];
-    so[lane] = incl - cnt;
-    const unsigned wave_pairs = __shfl(incl, 63, 64);
-    if (lane == 63) {
-        so[64] = wave_pairs;
-        s_wave_total[wave] = wave_pairs;
+    const unsigned block_pairs = __shfl(incl, 63, 64);
+    if (wave == 0) {
+        s_off[lane] = incl - cnt;
+        if (lane == 63) s_off[64] = block_pairs;
     }
     const unsigned long long deferred = __ballot((raw & kDeferred) != 0u);
     __syncthreads();
-    unsigned wave_base = 0;
+    unsigned block_base = 0;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-        wave_base += s_before[w];
-        if (w < wave) wave_base += s_wave_total[w];
-    }
-    const unsigned tile_off = wave_base + (incl - cnt);
-    if (!inline_redo && tile < ntiles) offsets[tile] = tile_off;
-    if (tile == ntiles - 1) {
-        const unsigned k = tile_off + cnt;
-        msg_words[0] = (unsigned)n;
-        msg_words[1] = k;
-        if (size_prefix) *size_prefix = (int)(8u + k * (unsigned)(4 * PW));
+    for (int w = 0; w < kWaves; ++w) block_base += s_before[w];
+    const unsigned tile_off = block_base + (incl - cnt);
+    if (wave == 0) {
+        if (!inline_redo && tile < ntiles) offsets[tile] = tile_off;
+        if (tile == ntiles - 1) {
+            const unsigned k = tile_off + cnt;
+            msg_words[0] = (unsigned)n;
+            msg_words[1] = k;
+            if (size_prefix) *size_prefix = (int)(8u + k * (unsigned)(4 * PW));
+        }
     }
 
     unsigned* const pairs = msg_words + 2;
     bool overflow = false;
-    for (unsigned p0 = 0; p0 < wave_pairs; p0 += 64 * kCopyUnroll) {
+    for (unsigned p0 = 0; p0 < block_pairs; p0 += kGatherBlock * kCopyUnroll) {
         unsigned src_idx[kCopyUnroll];
         bool live[kCopyUnroll];
 #pragma unroll
         for (int q = 0; q < kCopyUnroll; ++q) {
-            const unsigned p = p0 + q * 64 + lane;
-            live[q] = p < wave_pairs;
-            // owner: last tile of this wavefront whose exclusive offset is <= p.  Six fixed steps
+            const unsigned p = p0 + q * kGatherBlock + tid;
+            live[q] = p < block_pairs;
+            // owner: last tile of this block whose exclusive offset is <= p.  Six fixed steps
             // without branches, so that the searches of one round overlap their LDS reads.
             int lo = 0;
 #pragma unroll
             for (int step = 32; step > 0; step >>= 1)
-                lo += (so[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
+                lo += (s_off[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
             if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
-            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - so[lo]);
+            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - s_off[lo]);
         }
         unsigned v[kCopyUnroll][PW];
 #pragma unroll
@@ -392,7 +390,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
 #pragma unroll
         for (int q = 0; q < kCopyUnroll; ++q)
             if (live[q]) {
-                const long long dst_pos = (long long)wave_base + p0 + q * 64 + lane;
+                const long long dst_pos = (long long)block_base + p0 + q * kGatherBlock + tid;
                 if (dst_pos < cap_pairs) {
 #pragma unroll
                     for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
@@ -408,12 +406,14 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     if (inline_redo && deferred != 0ull) {
         const T thr = thr_ptr ? *thr_ptr : thr_val;
         unsigned long long todo = deferred;
+        int turn = 0;
         while (todo) {
             const int l = __ffsll((long long)todo) - 1;
             todo &= todo - 1;
             const unsigned pos = __shfl(tile_off, l, 64);
-            process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, first + l, lane, nullptr, nullptr, nullptr,
-                                                    0u, pairs, (long long)pos, cap_pairs, status);
+            if ((turn++ % kWaves) == wave)  // the block's wavefronts take the deferred tiles in turn
+                process_tile<T, MODE, VEC, ITEMS, true>(data, update, n, thr, first + l, lane, nullptr, nullptr,
+                                                        nullptr, 0u, pairs, (long long)pos, cap_pairs, status);
         }
     }
 }
@@ -482,7 +482,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
     // give the second pass the whole GPU instead of the gather kernel's few blocks
     const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
-    const unsigned gather_blocks = (ntiles + kGatherBlock - 1) / kGatherBlock;
+    const unsigned gather_blocks = (ntiles + kGatherTiles - 1) / kGatherTiles;
     hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
                        update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->block_sums,
                        h->tile_offsets, h->staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
