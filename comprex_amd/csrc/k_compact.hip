@@ -14,10 +14,10 @@
 //                    tile's count to counts[tile], and the residual is written back once
 //                    with survivors replaced by +0.  A tile with more survivors than its
 //                    slot holds does nothing but record its count with the "deferred" bit.
-//  2. gather_kernel  each 256-thread block adds up the per-block survivor sums the streaming
-//                    pass left for the tiles before its own 256, scans its own counts,
-//                    copies its staged slots to their final position in the message with
-//                    lane-contiguous stores (one wavefront per 64 tiles) and processes the few
+//  2. gather_kernel  each 256-thread block owns 64 tiles: it adds up the per-block survivor sums
+//                    the streaming pass left for the tiles before them, scans the 64 counts,
+//                    copies the staged slots to their final position in the message with
+//                    lane-contiguous stores (all its wavefronts together) and processes the few
 //                    deferred tiles it owns straight into their final position, which is known
 //                    by now; the last block writes the header.
 //  3. redo_kernel    launched only when the threshold is known to select (nearly) everything
