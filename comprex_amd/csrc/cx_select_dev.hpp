@@ -29,18 +29,20 @@ __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long l
     constexpr int kPer = kRadixBins / BLOCK;  // bins per thread
     const int t = threadIdx.x;
     const int hi = kRadixBins - 1 - t * kPer;  // thread t owns bins [hi - kPer + 1, hi], top digits first
+    // a vector holds fewer than 2^31 keys: 32-bit sums are exact, and half the cross-lane traffic
+    const unsigned want = rank > 0xffffffffull ? 0xffffffffu : (unsigned)rank;
     unsigned cnt[kPer];
-    unsigned long long local = 0;
+    unsigned local = 0;
 #pragma unroll
     for (int q = 0; q < kPer; ++q) {
         cnt[q] = hist[hi - q];
         local += cnt[q];
     }
-    unsigned long long incl = local;  // inclusive scan over threads
+    unsigned incl = local;  // inclusive scan over threads
     const int lane = t & 63, wave = t >> 6;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
-        const unsigned long long up = __shfl_up(incl, o, 64);
+        const unsigned up = __shfl_up(incl, o, 64);
         if (lane >= o) incl += up;
     }
     if (lane == 63) s_sum[wave] = incl;
@@ -49,13 +51,13 @@ __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long l
         *s_above = 0ull;
     }
     __syncthreads();
-    unsigned long long before = incl - local;
-    for (int w = 0; w < wave; ++w) before += s_sum[w];
-    if (rank >= before && rank < before + local) {
-        unsigned long long acc = before;
+    unsigned before = incl - local;
+    for (int w = 0; w < wave; ++w) before += (unsigned)s_sum[w];
+    if (want >= before && want - before < local) {
+        unsigned acc = before;
 #pragma unroll
         for (int q = 0; q < kPer; ++q) {
-            if (rank < acc + cnt[q]) {
+            if (want - acc < cnt[q]) {
                 *s_digit = (unsigned)(hi - q);
                 *s_above = acc;
                 break;
