@@ -96,6 +96,59 @@ int comprex_p2p_large() {
     return print_pass(errors);
 }
 
+// Conservation gold with a ThresholdTopK that samples caller-chosen positions (cloned into the
+// communicator by setThreshold), device-resident gradient.
+int comprex_p2p_sample_positions() {
+    typedef float data_t;
+    const int size = 200003, m = 5000, num_runs = 5;
+    std::vector<data_t> values(size), result(size, (data_t)0);
+    std::vector<int> pos(m);
+    unsigned x = 4242u;
+    for (int i = 0; i < size; ++i) {
+        x = x * 1664525u + 1013904223u;
+        values[i] = (data_t)((int)((x >> 8) % 20001u) - 10000);
+    }
+    for (int i = 0; i < m; ++i) {
+        x = x * 1664525u + 1013904223u;
+        pos[i] = (int)((x >> 8) % (unsigned)size);
+    }
+    GaspiEnvironment env(1 << 28);
+    ThresholdTopK<data_t> threshold(0.02f);
+    threshold.set_sample_positions(pos.data(), m);
+    std::vector<ComprEx<data_t> > cmprex;
+    cmprex.reserve(2);
+    for (int rank = 0; rank < 2; ++rank) {
+        env.set_rank(rank, 2);
+        cmprex.emplace_back(env.get_segment(), size, 3.0f, true);
+        cmprex[rank].setThreshold(threshold);
+        cmprex[rank].setCompressor(CompressorIndexPairs<data_t>());
+        cmprex[rank].connectTo((rank + 1) % 2, (rank + 1) % 2, 5);
+    }
+    void* d_values = nullptr;
+    cxx::check(cx_device_alloc(&d_values, (size_t)size * sizeof(data_t)));
+    cxx::Handle h;
+    cxx::check(cx_copy(h.get(), d_values, values.data(), (size_t)size * sizeof(data_t)));
+    int errors = 0;
+    for (int run = 0; run < num_runs; ++run) {
+        if (run < num_runs - 1) cmprex[0].writeRemote(static_cast<const data_t*>(d_values), size);
+        else cmprex[0].flushRests();
+        cmprex[1].readRemote_add(result.data(), size);
+        if (run == 0) {  // about two percent of the elements went out (the sample decides, not the vector)
+            long sent = 0;
+            for (int i = 0; i < size; ++i) sent += result[i] != 0;
+            if (sent < size / 100 || sent > size / 25) {
+                std::cout << "first message carried " << sent << " elements" << std::endl;
+                ++errors;
+            }
+        }
+    }
+    for (int i = 0; i < size; ++i)
+        if (result[i] != (data_t)(num_runs - 1) * values[i]) ++errors;
+    cx_device_free(d_values);
+    std::cout << "ComprEx point to point, caller-chosen sample positions, device gradient" << std::endl;
+    return print_pass(errors);
+}
+
 // Comprex_AllToOneAllreduce::apply / flush (reference src/allreduce.tpp:172-237), every rank's
 // part executed in the order the data dependencies impose.
 template <typename data_t> int all_to_one(const char* name, int numRanks, int size, int num_runs, float ratio) {
@@ -264,6 +317,7 @@ int main() {
     failed += comprex_p2p<float>("float");
     failed += comprex_p2p<double>("double");
     failed += comprex_p2p_large();
+    failed += comprex_p2p_sample_positions();
     failed += all_to_one<int>("int", 4, 1000, 10, 0.01f);
     failed += all_to_one<float>("float", 3, 100000, 5, 0.001f);
     failed += variants_and_forwarders<int>("int");
