@@ -97,7 +97,7 @@ def full_size(ref):
 
     ef_run("C1", W.C1, W.c1_gradient, W.C1["iters"])
     ef_run("C2", W.C2, W.c2_gradient, W.C2["iters"])
-    ef_run("C3", W.C3, W.c3_gradient, 3)  # first 3 of 20 iterations (each ~1 s of reference time)
+    ef_run("C3", W.C3, W.c3_gradient, W.C3["iters"])
 
     # C4: sampled (host-supplied indices are not a reference feature; the reference-faithful
     # strided default is) and exact

@@ -294,6 +294,39 @@ def test_write_remote_is_prepare_plus_compress(oracle, refimpl, send_size_bytes)
     assert (r0 == 0).all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_add_rests_is_elementwise_sum_in_the_same_type(oracle, dtype):
+    """comprEx.tpp:159-169 addRests: data[i] += rests[i], one addition per element in T.  Pinned by
+    what the arithmetic fixes: numpy's same-dtype sum (IEEE round-to-nearest for the float types,
+    wrap-free int sums), hand-picked fp32 cases where the sum rounds, and the mistakes a restatement
+    could make (swapped operands' sign, rests modified, one element too few, a wider accumulator)."""
+    rng = np.random.default_rng(11)
+    for n in (0, 1, 2, 7, 1000, 4099):
+        data = _rand(rng, n, dtype, 100.0)
+        rests = _rand(rng, n, dtype, 3.0)
+        want = (data + rests).astype(dtype)
+        d, r = data.copy(), rests.copy()
+        oracle.add_rests(d, r)
+        assert d.tobytes() == want.tobytes()
+        assert r.tobytes() == rests.tobytes(), "the residual itself is read-only here"
+        if n:
+            assert not np.array_equal(d, data - rests) or not rests.any()
+    if dtype == np.float32:
+        # sums that are not representable: 2^24 + 1 is a tie and rounds to even, 0.1f + 0.2f rounds in
+        # fp32, 1 + (2^-24 + 2^-47) lies just above the halfway point and rounds up
+        data = np.array([16777216.0, 0.1, 1.0, -0.0, 1e38, 1.0], np.float32)
+        rests = np.array([1.0, 0.2, 2.0 ** -24 + 2.0 ** -47, 0.0, 3e38, -1.0], np.float32)
+        d = data.copy()
+        oracle.add_rests(d, rests)
+        assert d[0] == np.float32(16777216.0) and d[1] == np.float32(0.1) + np.float32(0.2)
+        assert d[2] == np.nextafter(np.float32(1.0), np.float32(2.0))
+        assert d[3] == 0 and not np.signbit(d[3]) and np.isinf(d[4]) and d[5] == 0
+    if dtype == np.int32:
+        d = np.array([2147483000, -5, 7], np.int32)
+        oracle.add_rests(d, np.array([647, 5, -9], np.int32))
+        assert d.tolist() == [2147483647, 0, -2]
+
+
 def test_exact_mode_survivor_count(oracle):
     """Exact top-k sends ceil_f32(n*topK)-1 pairs when magnitudes are distinct:
     the threshold is the (pos+1)-th largest magnitude and selection is strict '>'."""
