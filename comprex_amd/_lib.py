@@ -58,6 +58,8 @@ def lib():
         "cx_topk_threshold_indexed": (i, [vp, i, vp, vp, i, vp, i, f, vp, vp]),
         "cx_threshold_slot": (vp, [vp]),
         "cx_ip_compress": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp, C.POINTER(i)]),
+        "cx_ip_compress_noalloc": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp]),
+        "cx_noalloc_max_elements": (ll, []),
         "cx_ip_compress_topk": (i, [vp, i, vp, ll, vp, vp, i, C.c_float, vp, vp, C.POINTER(i)]),
         "cx_get_option": (i, [vp, C.c_char_p, C.POINTER(i)]),
         "cx_rle_compress": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp, C.POINTER(i)]),

@@ -214,6 +214,12 @@ int cx_create(cx_handle* out, void* hip_stream) {
         cx_destroy(h);
         return fail(CX_ERR_HIP, "cx_create: %s", hipGetErrorString(e));
     }
+    // where this device keeps the static scratch array of cx_ip_compress_noalloc
+    const int rc = locate_static_scratch(&h->static_scratch);
+    if (rc != CX_OK) {
+        cx_destroy(h);
+        return rc;
+    }
     *out = h;
     return CX_OK;
 }
@@ -360,6 +366,16 @@ int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capaci
     if (!h) return fail(CX_ERR_INVALID, "null handle");
     CX_DISPATCH(dt, compress_impl<T>(h, out_msg, out_capacity, data, update, n, thr_host, d_thr, d_size_prefix, h_bytes));
 }
+
+int cx_ip_compress_noalloc(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data,
+                           void* update, int n, const void* thr_host, const void* d_thr, int* d_size_prefix) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    CX_DISPATCH(dt, launch_compact<T>(h, out_msg, out_capacity, static_cast<const T*>(data), static_cast<T*>(update), n,
+                                      static_cast<const T*>(thr_host), static_cast<const T*>(d_thr), d_size_prefix,
+                                      true));
+}
+
+long long cx_noalloc_max_elements(void) { return noalloc_max_elements(); }
 
 int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
                         int n, float topK, void* d_thr_out, int* d_size_prefix, int* h_bytes) {

@@ -94,6 +94,8 @@ struct cx_handle_s {
     unsigned epoch = 0;                // launch number
     unsigned parity = 0;               // flips with every full pass over the vectors: 1 = the next one walks from the end
 
+    unsigned* static_scratch = nullptr; // this device's copy of the library's static scratch array (not owned)
+
     unsigned* reduce_bounds = nullptr;  // tiled reduce: first pair of each message in each dense tile
     size_t reduce_bounds_cap = 0;
 
@@ -133,7 +135,10 @@ namespace cx {
 // ---- launchers implemented in the k_*.hip files -----------------------------
 template <typename T>
 int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
-                   const T* thr_host, const T* d_thr, int* d_size_prefix);
+                   const T* thr_host, const T* d_thr, int* d_size_prefix, bool no_alloc = false);
+// allocation-free variant: this device's copy of the static scratch array, and its size limit
+int locate_static_scratch(unsigned** out);
+long long noalloc_max_elements();
 
 template <typename T>
 int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m,

@@ -29,6 +29,8 @@
 #include "cx_common.hpp"
 #include "cx_select_dev.hpp"
 
+#include <mutex>
+
 namespace cx {
 
 namespace {
@@ -424,6 +426,27 @@ __global__ void empty_message_kernel(unsigned* msg_words, int n, int* size_prefi
     if (size_prefix) *size_prefix = 8;
 }
 
+// The compaction's scratch arrays: per-tile staging slots, counts, final offsets, per-block sums.
+struct Scratch {
+    unsigned* staging;
+    unsigned* counts;
+    unsigned* offsets;
+    unsigned* block_sums;
+};
+
+// ---- scratch of the allocation-free entry point (cx_ip_compress_noalloc) -------------------
+// One array per GPU, part of the code object, alive until the process ends.  Sized for vectors of
+// up to kNoAllocMaxN elements of any supported type and tile shape: staging needs at most 3/8 of a
+// 32-bit word per element (8-byte elements: 64 slots of 3 words per 512 elements), the smallest
+// tile has 256 elements.  Every launch writes what it later reads (counts, sums, slots), so stale
+// contents of an earlier call are harmless; two calls that overlap in time on one GPU would race.
+constexpr long long kNoAllocMaxN = 1ll << 24;
+constexpr size_t kStaticStagingWords = (size_t)kNoAllocMaxN * 3 / 8 + 1024;
+constexpr size_t kStaticTiles = (size_t)kNoAllocMaxN / 256 + 64;
+constexpr size_t kStaticSumsWords = kStaticTiles / 4 + 64;
+constexpr size_t kStaticWords = kStaticStagingWords + 2 * kStaticTiles + kStaticSumsWords;
+static __device__ __align__(256) unsigned scratch[kStaticWords];
+
 int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
     if (ntiles > h->tiles_cap) {
         size_t cap = h->tiles_cap ? h->tiles_cap : 4096;
@@ -454,13 +477,31 @@ int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
 
 template <typename T, int MODE, int VEC, int ITEMS>
 int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
-               long long cap_pairs, int* size_prefix, DeviceStatus* status) {
+               long long cap_pairs, int* size_prefix, DeviceStatus* status, bool no_alloc) {
     constexpr int kTile = 64 * VEC * ITEMS;
     constexpr int kCap = kTile / 8;
     constexpr int PW = Elem<T>::pair_words;
     const unsigned ntiles = (unsigned)(((long long)n + kTile - 1) / kTile);
-    int rc = ensure_scratch(h, ntiles, (size_t)ntiles * kCap * PW);
-    if (rc != CX_OK) return rc;
+    Scratch sc;
+    if (no_alloc) {
+        // the per-GPU static array, cut into the four arrays; never grows
+        unsigned* base = h->static_scratch;
+        if (!base) return fail(CX_ERR_INTERNAL, "compress: the static scratch array was not located on this device");
+        if ((size_t)ntiles * kCap * PW > kStaticStagingWords || (size_t)ntiles > kStaticTiles ||
+            (size_t)(ntiles + kWavesPerBlock - 1) / kWavesPerBlock > kStaticSumsWords)
+            return fail(CX_ERR_INVALID, "compress: %d elements exceed the static scratch array", n);
+        sc.staging = base;
+        sc.counts = base + kStaticStagingWords;
+        sc.offsets = sc.counts + kStaticTiles;
+        sc.block_sums = sc.offsets + kStaticTiles;
+    } else {
+        int rc = ensure_scratch(h, ntiles, (size_t)ntiles * kCap * PW);
+        if (rc != CX_OK) return rc;
+        sc.staging = h->staging;
+        sc.counts = h->tile_counts;
+        sc.offsets = h->tile_offsets;
+        sc.block_sums = h->block_sums;
+    }
     h->epoch += 1u;
     if (h->epoch == 0u) h->epoch = 1u;  // 0 is what a fresh flag holds
     unsigned* redo_flag = h->redo_flag;
@@ -476,7 +517,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
         CX_HIP(hipEventRecord(ev[0], h->stream));
     }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
-                       (long long)n, thr_ptr, thr_val, h->staging, h->tile_counts, h->block_sums, redo_flag, h->epoch, ntiles,
+                       (long long)n, thr_ptr, thr_val, sc.staging, sc.counts, sc.block_sums, redo_flag, h->epoch, ntiles,
                        reverse);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
@@ -484,13 +525,13 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
     const unsigned gather_blocks = (ntiles + kGatherTiles - 1) / kGatherTiles;
     hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
-                       update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->block_sums,
-                       h->tile_offsets, h->staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
+                       update, (long long)n, thr_ptr, thr_val, sc.counts, sc.block_sums,
+                       sc.offsets, sc.staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
                        status);
     if (dense_hint) {
         const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
         hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
-                           update, (long long)n, thr_ptr, thr_val, h->tile_counts, h->tile_offsets, redo_flag, h->epoch,
+                           update, (long long)n, thr_ptr, thr_val, sc.counts, sc.offsets, redo_flag, h->epoch,
                            ntiles, msg_words + 2, cap_pairs, status);
     }
     CX_HIP(hipGetLastError());
@@ -499,21 +540,47 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
 
 template <typename T, int VEC, int ITEMS>
 int launch_mode(cx_handle h, int mode, const T* data, T* update, int n, const T* thr_ptr, T thr_val,
-                unsigned* msg_words, long long cap_pairs, int* size_prefix) {
+                unsigned* msg_words, long long cap_pairs, int* size_prefix, bool no_alloc = false) {
     DeviceStatus* st = h->d_status;
-    if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
-    if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
-    if (mode == 2) return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
-    return launch_all<T, 3, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st);
+    if (mode == 0) return launch_all<T, 0, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st, no_alloc);
+    if (mode == 1) return launch_all<T, 1, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st, no_alloc);
+    if (mode == 2) return launch_all<T, 2, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st, no_alloc);
+    return launch_all<T, 3, VEC, ITEMS>(h, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, size_prefix, st, no_alloc);
 }
 
 }  // namespace
 
+// Address of this device's copy of the static scratch array.  The array's name is only a
+// host-side stand-in for the symbol; the address a kernel can use comes from the runtime, per
+// device, with that device current.
+int locate_static_scratch(unsigned** out) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex lock;
+    static unsigned* per_device[kMaxDevices];  // each GPU holds its own copy at its own address
+    *out = nullptr;
+    int device = 0;
+    CX_HIP(hipGetDevice(&device));
+    if (device < 0 || device >= kMaxDevices) return fail(CX_ERR_INVALID, "device ordinal %d not supported", device);
+    std::lock_guard<std::mutex> guard(lock);
+    if (!per_device[device]) {
+        void* p = nullptr;
+        CX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(CX_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+        per_device[device] = static_cast<unsigned*>(p);
+    }
+    *out = per_device[device];
+    return CX_OK;
+}
+
+long long noalloc_max_elements() { return kNoAllocMaxN; }
+
 template <typename T>
 int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
-                   const T* thr_host, const T* d_thr, int* d_size_prefix) {
+                   const T* thr_host, const T* d_thr, int* d_size_prefix, bool no_alloc) {
     constexpr int kPairBytes = 4 * Elem<T>::pair_words;
     if (!out_msg || n < 0) return fail(CX_ERR_INVALID, "compress: null message buffer or negative size");
+    if (no_alloc && (long long)n > kNoAllocMaxN)
+        return fail(CX_ERR_INVALID, "cx_ip_compress_noalloc: %d elements exceed the limit of %lld", n, kNoAllocMaxN);
     if ((reinterpret_cast<uintptr_t>(out_msg) & 3u) != 0)
         return fail(CX_ERR_INVALID, "compress: message buffer must be 4-byte aligned");
     if (out_capacity < 8) return fail(CX_ERR_CAPACITY, "compress: message buffer smaller than its 8-byte header");
@@ -532,11 +599,11 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
     constexpr int kVec = 16 / (int)sizeof(T);
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(update)) & 15u) == 0;
     if (!vec_ok)  // sub-vectors at odd offsets: scalar loads, same tile order
-        return launch_mode<T, 1, 16>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+        return launch_mode<T, 1, 16>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix, no_alloc);
     switch (h->compact_items) {
-        case 2: return launch_mode<T, kVec, 2>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
-        case 4: return launch_mode<T, kVec, 4>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
-        case 8: return launch_mode<T, kVec, 8>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix);
+        case 2: return launch_mode<T, kVec, 2>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix, no_alloc);
+        case 4: return launch_mode<T, kVec, 4>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix, no_alloc);
+        case 8: return launch_mode<T, kVec, 8>(h, mode, data, update, n, thr_ptr, thr_val, msg_words, cap_pairs, d_size_prefix, no_alloc);
         default: return fail(CX_ERR_INVALID, "compress: unsupported compact_items %d", h->compact_items);
     }
 }
@@ -722,8 +789,8 @@ CX_INSTANTIATE_FUSED(double)
 CX_INSTANTIATE_FUSED(int)
 #undef CX_INSTANTIATE_FUSED
 
-template int launch_compact<float>(cx_handle, void*, long long, const float*, float*, int, const float*, const float*, int*);
-template int launch_compact<double>(cx_handle, void*, long long, const double*, double*, int, const double*, const double*, int*);
-template int launch_compact<int>(cx_handle, void*, long long, const int*, int*, int, const int*, const int*, int*);
+template int launch_compact<float>(cx_handle, void*, long long, const float*, float*, int, const float*, const float*, int*, bool);
+template int launch_compact<double>(cx_handle, void*, long long, const double*, double*, int, const double*, const double*, int*, bool);
+template int launch_compact<int>(cx_handle, void*, long long, const int*, int*, int, const int*, const int*, int*, bool);
 
 }  // namespace cx

@@ -139,6 +139,22 @@ int cx_ip_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capaci
                    const void* thr_host, const void* d_thr,
                    int* d_size_prefix, int* h_bytes);
 
+/* No counterpart in the reference.  cx_ip_compress for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same kernels, same message, residual and size prefix, but the compaction's scratch (staging
+ * slots, per-tile counts and offsets, per-block sums) lives in a static device array of about
+ * 26 MB that each GPU holds from the moment the library's code is loaded there until the process
+ * ends, instead of in buffers the handle grows on demand.  No hipMalloc, hipFree or other
+ * allocating call is made and the call never waits; the byte count is delivered through
+ * d_size_prefix and the message header only.  n may not exceed cx_noalloc_max_elements()
+ * (16 777 216, any element type): larger vectors are refused with CX_ERR_INVALID.  All handles on
+ * one GPU share that array: calls that overlap in time on one GPU (different streams) race;
+ * calls in stream order do not.  The handle itself (cx_create) is made beforehand. */
+int cx_ip_compress_noalloc(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity,
+                           const void* data, void* update, int n,
+                           const void* thr_host, const void* d_thr, int* d_size_prefix);
+long long cx_noalloc_max_elements(void);
+
 /* ComprEx<T>::writeRemote with a whole-vector ThresholdTopK (src/comprEx.tpp:176-191 calling
  * src/threshold.hxx:160-167 in its `n < subsamples` mode, :224-231, and src/compressor.hxx:44-51):
  * the exact top-k threshold of |update + data| and the fused compress_add_update of
