@@ -201,6 +201,7 @@ int cx_create(cx_handle* out, void* hip_stream) {
     cx_handle h = new cx_handle_s();
     h->stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e = hipGetDevice(&h->device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&h->cu_count, hipDeviceAttributeMultiprocessorCount, h->device);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->redo_flag), 256);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->sel), sizeof(SelectState));
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->d_status), 256);
@@ -282,6 +283,9 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->select_bracket = value ? 1 : 0;
     } else if (!strcmp(key, "reduce_variant")) {
         h->reduce_variant = value;
+    } else if (!strcmp(key, "reduce_blocks_per_cu")) {
+        if (value < 1 || value > 32) return fail(CX_ERR_INVALID, "reduce_blocks_per_cu must be 1..32");
+        h->reduce_blocks_per_cu = value;
     } else if (!strcmp(key, "fused_topk")) {
         h->fused_topk = value ? 1 : 0;
     } else if (!strcmp(key, "select_short_list")) {
@@ -299,6 +303,7 @@ int cx_get_option(cx_handle h, const char* key, int* value) {
     else if (!strcmp(key, "stage_alternate")) *value = h->stage_alternate;
     else if (!strcmp(key, "select_bracket")) *value = h->select_bracket;
     else if (!strcmp(key, "reduce_variant")) *value = h->reduce_variant;
+    else if (!strcmp(key, "reduce_blocks_per_cu")) *value = h->reduce_blocks_per_cu;
     else if (!strcmp(key, "fused_topk")) *value = h->fused_topk;
     else if (!strcmp(key, "select_short_list")) *value = h->select_short_list;
     else if (!strcmp(key, "fused_topk_taken")) *value = h->fused_topk_taken;

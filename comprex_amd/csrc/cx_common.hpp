@@ -127,7 +127,10 @@ struct cx_handle_s {
     int select_short_list = 1;         // 1 = the two-launch select passes a short list of top keys to its second launch
     int fused_topk = 1;                // 1 = cx_ip_compress_topk may take its single-pass route
     int fused_topk_taken = 0;          // how the last cx_ip_compress_topk ran: 0 two calls, 1 single pass, 2 single pass abandoned
-    int reduce_variant = 0;            // 0 = tiled rank-ordered, 1 = per-message scatter
+    int reduce_variant = 0;            // 0 = rank-ordered, kernel chosen by message count; 1 = per-message scatter;
+                                       // 2 = always one block per tile behind a bounds pass; 3 = always the pipelined kernel
+    int reduce_blocks_per_cu = 1;      // persistent blocks per compute unit of the merged reduce
+    int cu_count = 0;                  // compute units of the device
 };
 
 namespace cx {

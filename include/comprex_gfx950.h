@@ -198,8 +198,8 @@ int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, i
 
 /* The chief's reduce loop of Comprex_AllToOneAllreduce::apply (src/allreduce.tpp:183-189):
  * out (+)= sum over messages in the order given.  `msgs` is a HOST array of n_msgs device
- * pointers.  accumulate == 0 starts from zero (decompress of the first message followed by
- * add of the rest), != 0 adds into `out`.  mode 0 = rank-ordered, bit-exact; mode 1 =
+ * pointers.  accumulate == 0 starts from zeros (every message is added, the first one to
+ * 0), != 0 adds into `out`.  mode 0 = rank-ordered, bit-exact; mode 1 =
  * floating-point atomics (order of additions unspecified). */
 int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* const* msgs, int n_msgs,
                  int accumulate, int mode);

@@ -485,7 +485,7 @@ def test_reduce_many_messages_duplicates_and_variants(dev, oracle):
     base = rng.standard_normal(n).astype(np.float32)
     gm = [_gpu(m) for m in msgs]
     try:
-        for variant in (0, 1):
+        for variant in (0, 1, 2, 3):
             dev.set_option("reduce_variant", variant)
             for accumulate in (False, True):
                 want = base.copy() if accumulate else np.zeros(n, np.float32)
@@ -500,6 +500,93 @@ def test_reduce_many_messages_duplicates_and_variants(dev, oracle):
             dev.decompress(g, gm[3])
             assert g.cpu().numpy().tobytes() == want.tobytes()
         dev.synchronize()
+    finally:
+        dev.set_option("reduce_variant", 0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pipelined_reduce_many_tiles_per_block_clusters_and_ragged_ends(dev, oracle, dtype):
+    """The pipelined rank-ordered reduce on vectors long enough that every block walks many tiles:
+    2..9 messages (more than one launch carries), pairs clustered so that far more than one chunk
+    of a message falls into one tile, long empty stretches, repeated indices, -0.0 values in the
+    first message (added to zeros), a vector that ends inside a tile, an output pointer
+    that is not 16-byte aligned, accumulate and overwrite: the checker's bits every time."""
+    rng = np.random.default_rng(99)
+    np_dt = np.dtype(dtype)
+    rec = np.dtype([("i", np.int32), ("v", np_dt)], align=False)
+    n = 6_000_011
+    try:
+        dev.set_option("reduce_variant", 3)
+        for n_msgs, unique in ((2, True), (5, False), (8, True), (9, False)):
+            msgs = []
+            for r in range(n_msgs):
+                parts = [rng.integers(0, n, 30_000)]
+                c0 = int(rng.integers(0, n - 5000))
+                parts.append(rng.integers(c0, c0 + 3000, 2500))          # a dense cluster: whole chunks in one tile
+                parts.append(np.arange(n - 700, n, 3))                    # the ragged end
+                if r == 1:
+                    parts = [rng.integers(n // 2, n // 2 + 100, 40)]      # a nearly empty message
+                idx = np.sort(np.concatenate(parts))
+                if unique:
+                    idx = np.unique(idx)
+                idx = idx.astype(np.int32)
+                body = np.empty(idx.size, rec)
+                body["i"] = idx
+                if np_dt.kind == "f":
+                    body["v"] = (rng.standard_normal(idx.size) * 10.0 ** rng.integers(-3, 4, idx.size)).astype(np_dt)
+                    if r == 0:
+                        body["v"][::7] = np_dt.type(-0.0)
+                else:
+                    body["v"] = rng.integers(-10**6, 10**6, idx.size).astype(np_dt)
+                msgs.append(np.concatenate([np.array([n, idx.size], np.int32).view(np.uint8), body.view(np.uint8)]))
+            gm = [_gpu(m) for m in msgs]
+            base = _rand(rng, n + 1, dtype)
+            for accumulate in (False, True):
+                for shift in (0, 1):  # shift 1: the output starts one element into an allocation
+                    say("pipelined reduce", np_dt.name, n_msgs, "messages, accumulate", accumulate, "shift", shift)
+                    want = base[shift:shift + n].copy() if accumulate else np.zeros(n, np_dt)
+                    for m in msgs:
+                        oracle.ip_add(m, want)
+                    g_all = _gpu(base)
+                    g = g_all[shift:shift + n]
+                    dev.reduce(g, gm, accumulate=accumulate, mode=0)
+                    dev.synchronize()
+                    assert g.cpu().numpy().tobytes() == want.tobytes()
+                    if shift == 0:
+                        assert g_all[n:].cpu().numpy().tobytes() == base[n:].tobytes(), "wrote past the vector"
+    finally:
+        dev.set_option("reduce_variant", 0)
+
+
+def test_pipelined_reduce_reports_unsorted_and_out_of_range(dev):
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rec = np.dtype([("i", np.int32), ("v", np.float32)])
+    n = 3_000_000
+    rng = np.random.default_rng(3)
+    good = np.unique(rng.integers(0, n, 20_000)).astype(np.int32)
+
+    def message(idx):
+        body = np.empty(idx.size, rec)
+        body["i"], body["v"] = idx, 1.0
+        return _gpu(np.concatenate([np.array([n, idx.size], np.int32).view(np.uint8), body.view(np.uint8)]))
+
+    swapped = good.copy()
+    swapped[[7000, 12000]] = swapped[[12000, 7000]]       # two pairs far apart trade places
+    beyond = np.concatenate([good, np.array([n + 5], np.int32)])
+    negative = np.concatenate([np.array([-3], np.int32), good])
+    try:
+        dev.set_option("reduce_variant", 3)
+        for bad in (swapped, beyond, negative):
+            g = torch.zeros(n, device="cuda")
+            dev.reduce(g, [message(good), message(bad)], accumulate=False, mode=0)
+            with pytest.raises(ComprexError) as e:
+                dev.synchronize()
+            assert e.value.code == _lib.CX_ERR_INDEX
+        g = torch.zeros(n, device="cuda")
+        dev.reduce(g, [message(good), message(good)], accumulate=False, mode=0)
+        dev.synchronize()
+        assert float(g.sum().item()) == 2.0 * good.size
     finally:
         dev.set_option("reduce_variant", 0)
 
