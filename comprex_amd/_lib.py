@@ -46,6 +46,7 @@ def lib():
         "cx_device_alloc": (i, [C.POINTER(vp), C.c_size_t]),
         "cx_device_free": (i, [vp]),
         "cx_copy": (i, [vp, vp, vp, C.c_size_t]),
+        "cx_copy_counted": (i, [vp, vp, vp, vp, ll]),
         "cx_create": (i, [C.POINTER(vp), vp]),
         "cx_destroy": (i, [vp]),
         "cx_set_stream": (i, [vp, vp]),

@@ -194,6 +194,11 @@ int cx_copy(cx_handle h, void* dst, const void* src, size_t bytes) {
     return CX_OK;
 }
 
+int cx_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    return launch_copy_counted(h, dst, src, d_bytes, capacity);
+}
+
 int cx_create(cx_handle* out, void* hip_stream) {
     if (!out) return fail(CX_ERR_INVALID, "cx_create: null output");
     *out = nullptr;

@@ -168,6 +168,7 @@ template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, cons
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);
 template <typename T>
 int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode);
+int launch_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity);
 template <typename T> int launch_zero(cx_handle h, T* v, int n);
 template <typename T> int launch_add_vec(cx_handle h, T* data, const T* rests, int n);
 template <typename T>

@@ -222,9 +222,12 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         for (int c = 0; c < VEC; ++c) {
             bool keep = (m >> c) & 1u;
             if (keep) {
-                if (pos < dst_limit) put_pair(dst + pos * PW, (unsigned)(e0 + c), s[j][c]);
-                else if (MODE == 3) keep = false;  // no room in the candidate list: stays in the residual
-                else overflow = true;
+                if (pos < dst_limit) {
+                    put_pair(dst + pos * PW, (unsigned)(e0 + c), s[j][c]);
+                } else {
+                    keep = false;  // no room in the message: stays in the residual (the header counts what was written)
+                    if (MODE != 3) overflow = true;
+                }
                 ++pos;
             }
             w.x[c] = keep ? (T)0 : s[j][c];
@@ -357,7 +360,10 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     if (wave == 0) {
         if (!inline_redo && tile < ntiles) offsets[tile] = tile_off;
         if (tile == ntiles - 1) {
-            const unsigned k = tile_off + cnt;
+            unsigned k = tile_off + cnt;
+            // never announce more pairs than the buffer holds (candidate lists keep the full count:
+            // their reader checks it against the capacity)
+            if (MODE != 3 && (long long)k > cap_pairs) k = (unsigned)cap_pairs;
             msg_words[0] = (unsigned)n;
             msg_words[1] = k;
             if (size_prefix) *size_prefix = (int)(8u + k * (unsigned)(4 * PW));
@@ -396,10 +402,10 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
                 if (dst_pos < cap_pairs) {
 #pragma unroll
                     for (int w = 0; w < PW; ++w) pairs[dst_pos * PW + w] = v[q][w];
-                } else if (MODE == 3) {
-                    update[v[q][0]] = pair_value<T>(v[q]);  // no room in the candidate list: back into the residual
                 } else {
-                    overflow = true;
+                    // no room in the message (or candidate list): the value goes back into the residual
+                    if (MODE != 2) update[v[q][0]] = pair_value<T>(v[q]);
+                    if (MODE != 3) overflow = true;
                 }
             }
     }
@@ -743,6 +749,7 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
 #pragma unroll
                 for (int q = 0; q < PW; ++q) pairs[(size_t)at * PW + q] = w[q];
             } else {
+                if (w[0] < (unsigned)n) update[w[0]] = pair_value<T>(w);  // no room in the message: stays in the residual
                 overflow = true;
             }
         }
@@ -751,6 +758,7 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
     }
     if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
     if (blockIdx.x == kFilterBlocks - 1 && tid == 0) {
+        if ((long long)pos > cap_pairs) pos = (unsigned)cap_pairs;  // never announce more than was written
         msg_words[0] = (unsigned)n;
         msg_words[1] = pos;
         if (size_prefix) *size_prefix = (int)(8u + pos * (unsigned)(4 * PW));

@@ -111,8 +111,8 @@ __global__ __launch_bounds__(kBlock) void rle_count_kernel(const unsigned* __res
     if (threadIdx.x == 0) block_counts[blockIdx.x] = s_cnt;
 }
 
-// Stores one int32 of the message if it fits; a message that does not fit is reported, its header
-// keeps the true counts.
+// Stores one int32 of the message if it fits; a message that does not fit is reported and then
+// replaced by an empty one (rle_overflow_kernel).
 __device__ __forceinline__ void put_word(unsigned* msg_words, long long word, long long cap_words, unsigned v,
                                          bool& overflow) {
     if (word < cap_words) msg_words[word] = v;
@@ -215,6 +215,40 @@ __global__ __launch_bounds__(kBlock) void rle_write_kernel(const unsigned* __res
         runs_before += chunk_total;
     }
     if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+}
+
+// A message that did not fit (result[0] = its true size > capacity): nothing of it may be taken
+// for a message, and nothing may be lost.  The pairs the first pass took out of `update` go back
+// (it cleared them, so storing restores the sums), and the buffer gets the empty message (one
+// "not sent" run over the vector) when it has room for that, whose size is then what is reported.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void rle_overflow_kernel(const unsigned* __restrict__ ip_words, T* __restrict__ update,
+                                                              int n, unsigned* __restrict__ msg_words, long long capacity,
+                                                              int* __restrict__ size_prefix, int* __restrict__ result) {
+    constexpr int PW = Elem<T>::pair_words;
+    if ((long long)result[0] <= capacity) return;
+    const unsigned k = ip_words[1];
+    if (update) {
+        for (unsigned j = blockIdx.x * kBlock + threadIdx.x; j < k; j += gridDim.x * kBlock) {
+            const unsigned* w = ip_words + 2 + (size_t)PW * j;
+            if (w[0] < (unsigned)n) store_words<T>(reinterpret_cast<unsigned*>(update + w[0]), load_words<T>(w + 1));
+        }
+    }
+    __threadfence();
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        int bytes = 0;
+        if (capacity >= 20) {
+            msg_words[0] = (unsigned)n;
+            msg_words[1] = 0u;
+            msg_words[2] = n > 0 ? 1u : 0u;
+            msg_words[3] = 0u;
+            msg_words[4] = (unsigned)n;
+            bytes = n > 0 ? 20 : 16;
+        }
+        if (size_prefix) *size_prefix = bytes;
+        // result[0] is read by the other blocks of this kernel: it keeps the true size (the host
+        // compares it with the capacity and reports CX_ERR_CAPACITY)
+    }
 }
 
 // ---- decode: prefix sums over the run lengths ---------------------------------------------
@@ -366,6 +400,8 @@ int launch_rle_compress(cx_handle h, void* out_msg, long long out_capacity, cons
                        msg_words, cap_words, d_size_prefix, d_result, h->d_status);
     hipLaunchKernelGGL((rle_write_kernel<T, true>), dim3(kConvBlocks), dim3(kBlock), 0, h->stream, ip_words, h->rle_scan, n,
                        msg_words, cap_words, d_size_prefix, d_result, h->d_status);
+    hipLaunchKernelGGL(rle_overflow_kernel<T>, dim3(kConvBlocks), dim3(kBlock), 0, h->stream, ip_words, update, n, msg_words,
+                       out_capacity, d_size_prefix, d_result);
     CX_HIP(hipGetLastError());
     return CX_OK;
 }

@@ -794,6 +794,37 @@ inline unsigned grid_for(long long work_items, long long per_thread) {
 
 }  // namespace
 
+// dst[0 .. min(*d_bytes, capacity)) = src[..]: the count is read on the device
+__global__ __launch_bounds__(kBlock) void copy_counted_kernel(unsigned char* __restrict__ dst,
+                                                              const unsigned char* __restrict__ src,
+                                                              const int* __restrict__ d_bytes, long long capacity,
+                                                              int words_ok) {
+    long long bytes = *d_bytes;
+    if (bytes < 0) bytes = 0;
+    if (bytes > capacity) bytes = capacity;
+    const long long stride = (long long)gridDim.x * kBlock;
+    const long long first = (long long)blockIdx.x * kBlock + threadIdx.x;
+    long long done = 0;
+    if (words_ok) {  // both pointers 4-byte aligned
+        const long long nwords = bytes / 4;
+        for (long long i = first; i < nwords; i += stride)
+            reinterpret_cast<unsigned*>(dst)[i] = reinterpret_cast<const unsigned*>(src)[i];
+        done = nwords * 4;
+    }
+    for (long long i = done + first; i < bytes; i += stride) dst[i] = src[i];
+}
+
+int launch_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity) {
+    if (!dst || !src || !d_bytes || capacity < 0) return fail(CX_ERR_INVALID, "copy_counted: bad arguments");
+    if (capacity == 0) return CX_OK;
+    const int words_ok = ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 3u) == 0 ? 1 : 0;
+    hipLaunchKernelGGL(copy_counted_kernel, dim3(grid_for(capacity / 4 + 1, 4)), dim3(kBlock), 0, h->stream,
+                       static_cast<unsigned char*>(dst), static_cast<const unsigned char*>(src), d_bytes, capacity,
+                       words_ok);
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
 template <typename T> int launch_zero(cx_handle h, T* v, int n) {
     if (n < 0 || (!v && n > 0)) return fail(CX_ERR_INVALID, "zero: bad arguments");
     if (n == 0) return CX_OK;

@@ -79,6 +79,23 @@ protected:
                                     thr, send_sizeBytes ? reinterpret_cast<int*>(src_address() + at) : nullptr, false);
     }
 
+    // Sends of the whole residual.  Messages that earlier sends had to cut short for lack of room
+    // are not an error (what they could not hold stayed in the residual and leaves now); other
+    // errors recorded by the compressor's kernels are.
+    void forgive_short_messages() {
+        const int st = compressor->device_status();
+        if (st != CX_OK && st != CX_ERR_CAPACITY) cxx::check(st);
+    }
+    // After the flush's message has been handed over: a flush that did not fit its buffer has sent
+    // what fitted, the rest is still in the residual, and the caller is told (the reference writes
+    // past its buffer here).
+    void report_flush(int st) {
+        if (st == CX_ERR_CAPACITY)
+            throw std::runtime_error("flushRests: the send buffer held only part of the residual, the rest stays in the "
+                                     "residual: flush again or increase size_factor!");
+        cxx::check(st);
+    }
+
     // residual += d_data with the entries above the threshold compressed into the message at
     // `d_target`: one fused call when the threshold is a whole-vector top-k and the compressor
     // has a path for it, else false (nothing done) and the caller takes the two steps.
@@ -147,9 +164,14 @@ public:
     // Sends the whole residual (no thresholding: every non-zero element) and clears it.
     virtual void flushRests() {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        forgive_short_messages();
         wait_for_room();
-        compress_into(0, rests(), nullptr, rests_size, false);
+        // as an update: what is sent leaves the residual, what found no room stays (the reference
+        // compresses the residual as data and clears it afterwards: the same message and residual)
+        compress_into(0, nullptr, rests(), rests_size, false);
+        const int st = compressor->device_status();
         srcBuff_data->post();
+        report_flush(st);
         resetRests();
     }
 
@@ -353,6 +375,10 @@ protected:
     // the half that holds the message of the previous call is what the receiver sees: it is
     // copied to the front of the channel when it is "sent"
     cxx::DeviceBuffer halves_;
+    // sizeBytes of the reference, one per half, kept on the device: every compressor writes its
+    // message's byte count there (int32), and sending copies exactly that many bytes without the
+    // host reading it
+    cxx::DeviceBuffer half_bytes_;
 
     using ComprEx<VarTYPE>::restsVect;
     using ComprEx<VarTYPE>::srcBuff_data;
@@ -366,28 +392,30 @@ protected:
     long long write_offset() const { return doublebuffer_offset * doublebuffer_phase; }
     void update_doublebuffer_phase() { doublebuffer_phase = (doublebuffer_phase + 1) % 2; }
     char* half(long long off) const { return static_cast<char*>(halves_.data()) + off; }
+    int* half_bytes(long long off) const { return static_cast<int*>(half_bytes_.data()) + (off == 0 ? 0 : 1); }
 
     void ensure_halves() {
         if (!halves_.data()) halves_.reserve((size_t)(2 * doublebuffer_offset > 32 ? 2 * doublebuffer_offset : 32));
+        if (!half_bytes_.data()) {
+            half_bytes_.reserve(2 * sizeof(int));
+            cxx::check(cx_zero(this->handle_.get(), CX_I32, half_bytes_.data(), 2));
+        }
     }
 
     // "initTransferPart(sizeBytes, send_offset)": hand the half at `off` to the receiver
     void send_half(long long off) {
         cx_handle h = this->handle_.get();
         this->wait_for_room();
-        // the message's own header tells its length; copy header first, then the pairs it announces
-        int hdr[2] = {0, 0};
-        cxx::check(cx_copy(h, hdr, half(off), 8));
-        const size_t bytes = 8 + (size_t)(hdr[1] < 0 ? 0 : hdr[1]) * (4 + sizeof(VarTYPE));
-        cxx::check(cx_copy(h, this->src_address(), half(off), bytes));
+        const long long room = doublebuffer_offset < this->bufferSize ? doublebuffer_offset : this->bufferSize;
+        cxx::check(cx_copy_counted(h, this->src_address(), half(off), half_bytes(off), room));
         srcBuff_data->post();
     }
 
     void compress_half(long long off, const VarTYPE* d_data, VarTYPE* d_update, int n, bool use_threshold) {
         const VarTYPE* d_thr = use_threshold ? this->threshold->device_threshold() : nullptr;
         const VarTYPE thr = use_threshold && !d_thr ? this->threshold->get_threshold() : (VarTYPE)0;
-        this->compressor->compress_device(half(off), doublebuffer_offset, d_data, d_update, n, d_thr, thr, nullptr,
-                                          false);
+        this->compressor->compress_device(half(off), doublebuffer_offset, d_data, d_update, n, d_thr, thr,
+                                          half_bytes(off), false);
     }
 
 public:
@@ -395,7 +423,9 @@ public:
 
     FastComprEx(GaspiEnvironment* segment, int size, float size_factor = 1.0)
         : ComprEx<VarTYPE>(segment, size, size_factor * 2), doublebuffer_phase(0), is_first(true) {
-        doublebuffer_offset = (long long)((float)size * size_factor * (float)sizeof(VarTYPE));
+        // (int)(size * size_factor * sizeof(T)) in the reference; cut to a multiple of four bytes so that
+        // the second half starts where a message may start
+        doublebuffer_offset = (long long)((float)size * size_factor * (float)sizeof(VarTYPE)) & ~3ll;
     }
 
     FastComprEx(const FastComprEx<VarTYPE>& other) : ComprEx<VarTYPE>() { *this = other; }
@@ -411,19 +441,19 @@ public:
     virtual void flushRests() {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         ensure_halves();
+        this->forgive_short_messages();
         const long long so = send_offset();
-        if (is_first) {
-            // nothing compressed yet: the half is undefined in the reference (it adds whatever the
-            // buffer holds); an empty message is what a fresh buffer of zeros decodes to
-            compress_half(so, nullptr, nullptr, this->rests_size, false);
-        }
-        // the message that was compressed but never sent goes back into the residual ...
-        this->compressor->add_device(this->rests(), this->rests_size, half(so));
+        // the message that was compressed but never sent goes back into the residual (when nothing
+        // waits, the reference adds whatever its buffer holds: fresh memory, or the previous flush's
+        // message a second time; nothing is added here) ...
+        if (!is_first) this->compressor->add_device(this->rests(), this->rests_size, half(so));
         // ... and the whole residual is sent
-        compress_half(so, this->rests(), nullptr, this->rests_size, false);
+        compress_half(so, nullptr, this->rests(), this->rests_size, false);
+        const int st = this->compressor->device_status();
         send_half(so);
-        ComprEx<VarTYPE>::resetRests();
         is_first = true;
+        this->report_flush(st);
+        ComprEx<VarTYPE>::resetRests();
     }
 
     virtual void resetRests() {
@@ -443,7 +473,7 @@ public:
         }
         send_half(so);  // the message of the previous call
         cxx::Staged<const VarTYPE> v(h, this->stage_, vector, (size_t)size, true, false);
-        if (this->fused_topk_into(half(wo), doublebuffer_offset, v.get(), size, nullptr)) {
+        if (this->fused_topk_into(half(wo), doublebuffer_offset, v.get(), size, half_bytes(wo))) {
             update_doublebuffer_phase();
             return;
         }
@@ -487,10 +517,12 @@ public:
         }
         send_half(so);
         if (!other->is_first) {
-            int hdr[2] = {0, 0};
-            cxx::check(cx_copy(h, hdr, other->half(other->send_offset()), 8));
-            const size_t bytes = 8 + (size_t)(hdr[1] < 0 ? 0 : hdr[1]) * (4 + sizeof(VarTYPE));
-            cxx::check(cx_copy(h, half(wo), other->half(other->send_offset()), bytes));
+            // memcpy(..., other->sizeBytes) and sizeBytes = other->sizeBytes, both on the device
+            const long long oso = other->send_offset();
+            const long long room = doublebuffer_offset < other->doublebuffer_offset ? doublebuffer_offset
+                                                                                  : other->doublebuffer_offset;
+            cxx::check(cx_copy_counted(h, half(wo), other->half(oso), other->half_bytes(oso), room));
+            cxx::check(cx_copy(h, half_bytes(wo), other->half_bytes(oso), sizeof(int)));
         } else {
             this->is_first = true;
         }

@@ -54,6 +54,15 @@ public:
 
     virtual Compressor<VarTYPE>* clone() const = 0;
 
+    // Not in the reference: bytes of the largest message a vector of n elements can produce.
+    virtual long long max_message_bytes(int n) const = 0;
+
+    // Not in the reference: waits for this compressor's GPU work and returns (and forgets) the first
+    // error a kernel recorded since the last call, CX_OK if none.  A message cut short for lack of
+    // room (CX_ERR_CAPACITY) is valid as far as it goes; what it could not hold stayed in the
+    // update vector.
+    virtual int device_status() { return cx_synchronize(handle_.get()); }
+
     // Device-side entry used by ComprEx: all pointers are device pointers, `capacity` is the
     // size of d_target in bytes, the threshold comes from d_threshold (device) or, when that is
     // NULL, from `threshold`.  d_size_prefix (may be NULL) receives the message's byte count.
@@ -100,7 +109,7 @@ public:
 
     virtual Compressor<VarTYPE>* clone() const { return new CompressorIndexPairs<VarTYPE>(*this); }
 
-    static long long max_message_bytes(int n) { return 8 + (long long)n * (4 + (long long)sizeof(VarTYPE)); }
+    virtual long long max_message_bytes(int n) const { return 8 + (long long)n * (4 + (long long)sizeof(VarTYPE)); }
 
     virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
                                 const VarTYPE* d_threshold, VarTYPE threshold, int* d_size_prefix, bool wait) {
@@ -210,7 +219,7 @@ public:
     virtual Compressor<VarTYPE>* clone() const { return new CompressorRLE<VarTYPE>(*this); }
 
     // n values, n + 1 run lengths at most
-    static long long max_message_bytes(int n) { return 16 + (long long)n * (long long)sizeof(VarTYPE) + 4ll * ((long long)n + 1); }
+    virtual long long max_message_bytes(int n) const { return 16 + (long long)n * (long long)sizeof(VarTYPE) + 4ll * ((long long)n + 1); }
 
     virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
                                 const VarTYPE* d_threshold, VarTYPE threshold, int* d_size_prefix, bool wait) {
@@ -297,6 +306,7 @@ public:
     CompressorNone() {}
     CompressorNone(const CompressorNone<VarTYPE>& other) : Compressor<VarTYPE>(other) {}
     virtual Compressor<VarTYPE>* clone() const { return new CompressorNone<VarTYPE>(*this); }
+    virtual long long max_message_bytes(int n) const { return 4 + (long long)n * (long long)sizeof(VarTYPE); }
 
     virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
                                 const VarTYPE*, VarTYPE, int* d_size_prefix, bool) {

@@ -67,6 +67,12 @@ int cx_device_alloc(void** out, size_t bytes);
 int cx_device_free(void* p);
 int cx_copy(cx_handle h, void* dst, const void* src, size_t bytes);
 
+/* No counterpart in the reference, whose transports take a host-side byte count
+ * (initTransferPart(sizeBytes, offset), src/comprEx.tpp:442): copies *d_bytes bytes (a device
+ * int32, e.g. the size prefix a compressor wrote; clamped to [0, capacity]) from src to dst, device
+ * memory both, in stream order, without the host ever reading the count. */
+int cx_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity);
+
 /* A handle owns one HIP stream reference and the scratch memory of one compressor
  * clone (tile descriptors, histograms, a device-side threshold slot, a status word).
  * It replaces the per-object state of Compressor<T>/ThresholdFunction<T> clones

@@ -15,6 +15,8 @@
  *   src/compressor.hxx:158-532  CompressorRLE (decoder and adder as they are; the encoder with its
  *                               value-index bug corrected, see cxo_rle_compress)
  *   src/comprEx.tpp:121-246     residual maintenance, writeRemote*, flushRests, readRemote*
+ *   src/comprEx.tpp:366-493     FastComprEx (one-call-stale sends from a double buffer)
+ *   src/compressor.hxx:83-151   CompressorNone
  *
  * Every function is pinned (tests/test_oracle_*.py) against: the compiled
  * reference headers (oracle/_ref, when the reference tree is present), the
@@ -118,6 +120,24 @@ int cxo_sample_count(int n, int subsamples);
     /* comprEx.tpp:128-142 flushRests: data-only compress of rests at threshold 0, then       \
      * zero the residual. */                                                                  \
     int cxo_flush_rests_##SFX(void* buf, int send_size_bytes, T* rests, int n);
+
+/* CompressorNone (compressor.hxx:83-151) and FastComprEx (comprEx.tpp:366-493); see the .inc. */
+#define CXO_DECLARE_FAST(SFX, T)                                                                       \
+    int cxo_none_compress_##SFX(void* out, const T* data, T* update, int n);                           \
+    int cxo_none_decompress_##SFX(T* out, int out_n, const void* in);                                  \
+    int cxo_none_add_##SFX(T* out, int out_n, const void* in);                                         \
+    int cxo_fast_write_remote_##SFX(int codec, T* rests, int n, const T* vec, unsigned char* halves,   \
+                                    int half_bytes, int* st, T* thr, float topK, int default_subsamples, \
+                                    float subsample_factor, unsigned char* sent);                      \
+    int cxo_fast_flush_rests_##SFX(int codec, T* rests, int n, unsigned char* halves, int half_bytes,  \
+                                   int* st, unsigned char* sent);                                      \
+    int cxo_fast_write_remote_same_as_##SFX(int codec, T* rests, int n, unsigned char* halves,         \
+                                            int half_bytes, int* st, T thr,                            \
+                                            const unsigned char* other_halves, const int* other_st,    \
+                                            unsigned char* sent);
+CXO_DECLARE_FAST(f32, float)
+CXO_DECLARE_FAST(f64, double)
+CXO_DECLARE_FAST(i32, int)
 
 CXO_DECLARE(f32, float)
 CXO_DECLARE(f64, double)

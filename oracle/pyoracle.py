@@ -202,6 +202,37 @@ class Oracle:
         if r < 0:
             raise RuntimeError("Decompression vector size is bigger than output buffer!")
 
+    # ---- dense codec ---------------------------------------------------
+    def none_compress(self, data, update):
+        """CompressorNone: int32 n, then the values (update is modified in place)."""
+        ref_arr = data if data is not None else update
+        s = self._sfx(ref_arr)
+        out = np.zeros(4 + ref_arr.size * ref_arr.itemsize, dtype=np.uint8)
+        nbytes = self._f("none_compress_" + s, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int)(
+            _ptr(out), _ptr(data), _ptr(update), ref_arr.size)
+        return out[:nbytes]
+
+    def none_decompress(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("none_decompress_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(_ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+        return r
+
+    def none_add(self, msg, out):
+        s = self._sfx(out)
+        msg = np.ascontiguousarray(msg, dtype=np.uint8)
+        r = self._f("none_add_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p)(_ptr(out), out.size, _ptr(msg))
+        if r < 0:
+            raise RuntimeError("Decompression vector size is bigger than output buffer!")
+
+    def fast_comprex(self, n, dtype, codec="ip", size_factor=3.0, topK=0.01, default_subsamples=1000,
+                     subsample_factor=10.0):
+        """A FastComprEx sender (restatement only): see FastChannel."""
+        assert not self.ref
+        return FastChannel(self, n, dtype, codec, size_factor, topK, default_subsamples, subsample_factor)
+
     # ---- channel level (restatement only) ----------------------------
     def add_rests(self, data, rests):
         assert not self.ref
@@ -240,6 +271,48 @@ class Oracle:
         nbytes = self._f("flush_rests_" + s, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int)(
             _ptr(buf), int(send_size_bytes), _ptr(rests), rests.size)
         return buf[:nbytes + (4 if send_size_bytes else 0)]
+
+
+class FastChannel:
+    """Sender side of FastComprEx (comprEx.tpp:366-493) on the restatement: residual, the two
+    halves of the send buffer, sizeBytes / phase / is_first and the threshold's current value.
+    Every call returns the bytes it hands to the transport."""
+    CODECS = {"ip": 0, "rle": 1, "none": 2}
+
+    def __init__(self, oracle, n, dtype, codec, size_factor, topK, ds, sf):
+        self.o, self.n, self.dt, self.codec = oracle, n, np.dtype(dtype), self.CODECS[codec]
+        self.s = _SFX[self.dt]
+        self.rests = np.zeros(n, self.dt)
+        # doublebuffer_offset of the reference is size*size_factor*sizeof(T); the restatement's
+        # buffers are sized for the largest message of any codec
+        self.half_bytes = max(int(n * size_factor * self.dt.itemsize), 64 + n * (8 + self.dt.itemsize))
+        self.halves = np.zeros(2 * self.half_bytes, np.uint8)
+        self.st = np.array([0, 0, 1], np.int32)  # sizeBytes, phase, is_first
+        self.thr = _CT[self.s](0)
+        self.topK, self.ds, self.sf = topK, ds, sf
+
+    def write_remote(self, vec):
+        sent = np.zeros(self.half_bytes, np.uint8)
+        nb = self.o._f("fast_write_remote_" + self.s, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                       C.c_int, C.c_void_p, C.c_void_p, C.c_float, C.c_int, C.c_float, C.c_void_p)(
+            self.codec, _ptr(self.rests), self.n, _ptr(vec), _ptr(self.halves), self.half_bytes, _ptr(self.st),
+            C.byref(self.thr), self.topK, self.ds, self.sf, _ptr(sent))
+        return sent[:nb]
+
+    def flush_rests(self):
+        sent = np.zeros(self.half_bytes, np.uint8)
+        nb = self.o._f("fast_flush_rests_" + self.s, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
+                       C.c_void_p, C.c_void_p)(
+            self.codec, _ptr(self.rests), self.n, _ptr(self.halves), self.half_bytes, _ptr(self.st), _ptr(sent))
+        return sent[:nb]
+
+    def write_remote_same_as(self, other):
+        sent = np.zeros(self.half_bytes, np.uint8)
+        nb = self.o._f("fast_write_remote_same_as_" + self.s, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p,
+                       C.c_int, C.c_void_p, _CT[self.s], C.c_void_p, C.c_void_p, C.c_void_p)(
+            self.codec, _ptr(self.rests), self.n, _ptr(self.halves), self.half_bytes, _ptr(self.st), self.thr,
+            _ptr(other.halves), _ptr(other.st), _ptr(sent))
+        return sent[:nb]
 
 
 def parse_message(msg, dtype):

@@ -113,6 +113,31 @@ int cxr_calc_subsamples(float topK, int default_subsamples, float subsample_fact
         catch (const std::runtime_error&) { return -1; }                                          \
         return 0;                                                                                 \
     }
+/* the reference's dense codec (compressor.hxx:83-151) */
+#define CXR_DEFINE_NONE(SFX, T)                                                                   \
+    int cxr_none_compress_##SFX(void* out, const T* data, T* update, int n) {                     \
+        CompressorNone<T> c;                                                                      \
+        try {                                                                                     \
+            if (data && update) return c.compress_add_update(out, update, n, data, n, (T)0);      \
+            if (update) return c.compress_update(out, update, n, (T)0);                           \
+            return c.compress(out, data, n, (T)0);                                                \
+        } catch (const std::runtime_error&) { return -1; }                                        \
+    }                                                                                             \
+    int cxr_none_decompress_##SFX(T* out, int out_n, const void* in) {                            \
+        CompressorNone<T> c;                                                                      \
+        try { return c.decompress(out, out_n, in); }                                              \
+        catch (const std::runtime_error&) { return -1; }                                          \
+    }                                                                                             \
+    int cxr_none_add_##SFX(T* out, int out_n, const void* in) {                                   \
+        CompressorNone<T> c;                                                                      \
+        try { c.add(out, out_n, in); }                                                            \
+        catch (const std::runtime_error&) { return -1; }                                          \
+        return 0;                                                                                 \
+    }
+CXR_DEFINE_NONE(f32, float)
+CXR_DEFINE_NONE(f64, double)
+CXR_DEFINE_NONE(i32, int)
+
 CXR_DEFINE_RLE(f32, float)
 CXR_DEFINE_RLE(f64, double)
 CXR_DEFINE_RLE(i32, int)

@@ -158,7 +158,40 @@ def test_compress_capacity_and_size_errors(dev):
     with pytest.raises(ComprexError) as e:
         dev.compress(small, d, u, thr=0.5)
     assert e.value.code == _lib.CX_ERR_CAPACITY
-    assert small[:8].view(torch.int32).tolist() == [1000, 1000]  # header reports the true count
+    # the header announces what was written, and what found no room is still in the residual
+    assert small[:8].view(torch.int32).tolist() == [1000, 10]
+    pairs = small[8:].view(torch.int32).view(-1, 2)
+    assert pairs[:, 0].tolist() == list(range(10)) and small[8:].view(torch.float32).view(-1, 2)[:, 1].tolist() == [1.0] * 10
+    assert u[:10].tolist() == [0.0] * 10 and u[10:].tolist() == [1.0] * 990
+    big = _msgbuf(1000, np.float32)
+    assert dev.compress(big, None, u, thr=0.5) == 8 + 8 * 990 and not bool(u.any())
+    # the same through every route that places pairs: tiles deferred for their density (threshold 0:
+    # the write pass of a flush), the single-call exact top-k, and the run-length codec
+    for n, route in ((50_000, "flush"), (1 << 23, "topk"), (5000, "rle")):
+        rng = np.random.default_rng(8)
+        g_h = rng.integers(1, 100, n).astype(np.float32) * rng.choice([-1.0, 1.0], n).astype(np.float32)
+        r_h = rng.integers(-20, 20, n).astype(np.float32)
+        g, r = _gpu(g_h), _gpu(r_h)
+        tiny = torch.zeros(8 + 8 * 100, dtype=torch.uint8, device="cuda")
+        with pytest.raises(ComprexError) as e:
+            if route == "flush":
+                dev.compress(tiny, g, r, thr=0.0)
+            elif route == "topk":
+                dev.compress_topk(tiny, g, r, np.float32(0.001))
+            else:
+                dev.rle_compress(tiny, g, r, thr=1.0)
+        assert e.value.code == _lib.CX_ERR_CAPACITY, route
+        total = r_h + g_h
+        if route == "rle":  # cannot be cut short: an empty message, everything stays behind
+            assert tiny[:20].view(torch.int32).tolist() == [n, 0, 1, 0, n]
+            sent = np.zeros(n, np.float32)
+        else:
+            hdr = tiny[:8].view(torch.int32).tolist()
+            assert hdr[0] == n and 0 < hdr[1] <= 100
+            sent = torch.zeros(n, device="cuda")
+            dev.add(sent, tiny)
+            sent = sent.cpu().numpy()
+        assert np.array_equal(sent + r.cpu().numpy(), total), route  # nothing lost, nothing sent twice
     with pytest.raises(ComprexError) as e:
         dev.compress(_msgbuf(1000, np.float32), d, u[:999], thr=0.5)
     assert e.value.code == _lib.CX_ERR_SIZE_MISMATCH
@@ -297,9 +330,13 @@ def test_fused_exact_topk_message_buffer_too_small_and_bad_arguments(dev, oracle
     assert e.value.code == _lib.CX_ERR_CAPACITY
     assert dev.get_option("fused_topk_taken") == 1
     got = buf.cpu().numpy()
-    assert got[:8].tobytes() == want_msg[:8].tobytes()          # header keeps the true count
+    assert got[:8].view(np.int32).tolist() == [n, 1000]         # the header announces what was written
     assert got[8:].tobytes() == want_msg[8:keep].tobytes()      # the pairs that fit
-    assert gu.cpu().numpy().tobytes() == uu.tobytes()           # residual as after a full compress
+    # what found no room is still in the residual: the sums of the pairs that were not written
+    left = uu.copy()
+    rest = want_msg[keep:].view(np.dtype([("i", np.int32), ("v", np.float32)]))
+    left[rest["i"]] = rest["v"]
+    assert gu.cpu().numpy().tobytes() == left.tobytes()
     with pytest.raises(ComprexError) as e:
         dev.compress_topk(_msgbuf(n, np.float32), gd, gu, 1.5)
     assert e.value.code == _lib.CX_ERR_TOPK

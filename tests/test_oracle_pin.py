@@ -414,3 +414,101 @@ def test_rle_messages_decode_with_the_reference_decoder(oracle, refimpl, dtype):
                 assert acc[:n].tobytes() == (np.arange(n).astype(dtype) + want).astype(dtype).tobytes()
                 with pytest.raises(RuntimeError):
                     impl.rle_decompress(msg, np.zeros(n - 1, dtype))
+
+
+# ---------------------------------------------------------------- dense codec, FastComprEx
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_none_codec_matches_ref(oracle, refimpl, dtype):
+    """CompressorNone (compressor.hxx:83-151) against the compiled reference in its three modes;
+    its adder only on full-length messages (the reference's reads past a shorter one)."""
+    rng = np.random.default_rng(31)
+    for n in (1, 5, 1000):
+        d, u = _rand(rng, n, dtype), _rand(rng, n, dtype)
+        for data, update in ((d, u), (None, u), (d, None)):
+            u0 = None if update is None else update.copy()
+            u1 = None if update is None else update.copy()
+            m0 = oracle.none_compress(data, u0)
+            m1 = refimpl.none_compress(data, u1)
+            assert m0.tobytes() == m1.tobytes() and m0.size == 4 + n * np.dtype(dtype).itemsize
+            if update is not None:
+                assert u0.tobytes() == u1.tobytes() and not u0.any()
+            o0, o1 = _rand(rng, n + 3, dtype), None
+            o1 = o0.copy()
+            assert oracle.none_decompress(m0, o0) == refimpl.none_decompress(m0, o1) == m0.size
+            assert o0.tobytes() == o1.tobytes()
+            a0 = _rand(rng, n, dtype)
+            a1 = a0.copy()
+            oracle.none_add(m0, a0)
+            refimpl.none_add(m0, a1)
+            assert a0.tobytes() == a1.tobytes()
+    for impl in (oracle, refimpl):  # a message longer than the output is refused by both
+        with pytest.raises(RuntimeError):
+            impl.none_decompress(m0, np.zeros(n - 1, dtype))
+        with pytest.raises(RuntimeError):
+            impl.none_add(m0, np.zeros(n - 1, dtype))
+
+
+def test_fast_comprex_is_the_reference_calls_one_step_late(oracle, refimpl):
+    """comprEx.tpp:404-448 composed from the compiled reference's own threshold and compressor calls,
+    line by line, against the restated state machine: what leaves at call i is what call i-1
+    compressed (an empty message at the first call), a flush returns the unsent message to the
+    residual before it sends everything."""
+    rng = np.random.default_rng(41)
+    n, topk = 5000, np.float32(0.02)
+    fast = oracle.fast_comprex(n, np.float32, "ip", topK=topk)
+    rests = np.zeros(n, np.float32)       # the reference side
+    halves = [np.zeros(0, np.uint8), np.zeros(0, np.uint8)]
+    phase, is_first, thr = 0, True, np.float32(0)
+    script = "WWWFWFFWW"
+    for step, op in enumerate(script):
+        if op == "W":
+            g = _rand(rng, n, np.float32)
+            got = fast.write_remote(g)
+            write, send = phase, (phase + 1) % 2
+            if is_first:                                                  # :436-440
+                halves[send] = refimpl.ip_compress(None, rests, thr)
+                is_first = False
+            want = halves[send]                                           # :442
+            thr = refimpl.topk_prepare_with(rests, g, topk)               # :444
+            halves[write] = refimpl.ip_compress(g, rests, thr)            # :446
+            phase = (phase + 1) % 2                                       # :447
+            if step == 0:
+                assert want.size == 8 and want[4:8].view(np.int32)[0] == 0, "the first message is empty"
+        else:
+            got = fast.flush_rests()
+            send = (phase + 1) % 2
+            if not is_first:
+                refimpl.ip_add(halves[send], rests)                       # :413
+            halves[send] = refimpl.ip_compress(rests, None, np.float32(0))  # :415
+            want = halves[send]                                           # :417
+            rests[:] = 0                                                  # :418
+            is_first = True                                               # :419
+        assert got.tobytes() == want.tobytes(), (step, op)
+        assert fast.rests.tobytes() == rests.tobytes(), (step, op)
+        assert float(fast.thr.value) == float(thr)
+
+
+@pytest.mark.parametrize("codec", ["ip", "rle", "none"])
+@pytest.mark.parametrize("dtype", [np.float32, np.int32])
+def test_fast_comprex_conserves_what_it_is_given(oracle, codec, dtype):
+    """Whatever the codec: the messages that leave (each one call late) plus the flush add up to the
+    inputs, exactly for integer-valued data (gold of test/comprex.cpp:73-75 applied to FastComprEx),
+    and writeRemote_sameAs hands on the other channel's waiting message unchanged."""
+    rng = np.random.default_rng(43)
+    n = 3000
+    add = {"ip": oracle.ip_add, "rle": oracle.rle_add, "none": oracle.none_add}[codec]
+    a = oracle.fast_comprex(n, dtype, codec, topK=np.float32(0.05))
+    b = oracle.fast_comprex(n, dtype, codec, topK=np.float32(0.05))
+    total, got_a, got_b = np.zeros(n, dtype), np.zeros(n, dtype), np.zeros(n, dtype)
+    for it in range(6):
+        g = rng.integers(-50, 50, n).astype(dtype)
+        total += g
+        waiting_before = None if a.st[2] else a.halves[a.half_bytes * ((a.st[1] + 1) % 2):][:a.st[0]].copy()
+        add(a.write_remote(g), got_a)
+        msg_b = b.write_remote_same_as(a)
+        add(msg_b, got_b)
+        if it >= 1:  # b sends, one call late, what was waiting in a when b last copied
+            assert msg_b.tobytes() == copied.tobytes()
+        copied = a.halves[a.half_bytes * ((a.st[1] + 1) % 2):][:a.st[0]].copy()
+    add(a.flush_rests(), got_a)
+    assert np.array_equal(got_a, total) and not a.rests.any()
