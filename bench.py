@@ -37,9 +37,38 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def event_ms(torch, fn, reps, between=None):
+    """Mean milliseconds of fn() from HIP events on torch's current stream (the stream the library
+    launches on here); `between` runs untimed before every repetition."""
+    e0 = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    e1 = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+    for i in range(reps):
+        if between is not None:
+            between()
+        e0[i].record()
+        fn()
+        e1[i].record()
+    torch.cuda.synchronize()
+    return float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
+
+
+def host_description():
+    """Core count and CPU model of the box the CPU legs run on."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"nproc": os.cpu_count(), "cpu_model": model}
+
+
 def cpu_baseline(g, idx, topk, seconds):
     """The same step on one host core: the compiled reference headers when their library
-    travelled with the tree, else the plain-C restatement."""
+    travelled with the tree, else the plain-C restatement.  Threshold (prepare) and compress are
+    timed separately, as the reference runs them as two calls."""
     from oracle.pyoracle import Oracle, ref_available
     impl = Oracle(ref=True) if ref_available() else Oracle()
     n = g.size
@@ -51,17 +80,47 @@ def cpu_baseline(g, idx, topk, seconds):
         t0 = time.perf_counter()
         sums = rests[idx] + g[idx]                       # prep_add_vec's gather on the chosen positions
         thr = impl.calc_threshold(sums, topk)            # calc_threshold (nth_element)
+        t1 = time.perf_counter()
         msg = impl.ip_compress(g, rests, thr)            # compress_add_update
-        dt = time.perf_counter() - t0
+        t2 = time.perf_counter()
         k = int(msg[4:8].view(np.int32)[0])
         if it > 0:  # first pass is the warm-up
-            times.append((dt, 12 * n + 8 * k + 8 + 8 * idx.size))
+            times.append((t2 - t0, 12 * n + 8 * k + 8 + 8 * idx.size, t1 - t0, t2 - t1))
         it += 1
     med = sorted(times)[len(times) // 2]
-    return dict(value=med[1] / med[0] / 1e9, unit="GB/s", cores=1, kind=impl.kind,
-                sample="%d full steps (n=%d, %d sample positions) after 1 warm-up, median; %.1f ms/step"
-                       % (len(times), n, idx.size, med[0] * 1e3),
-                ms_per_step=med[0] * 1e3)
+    out = dict(value=med[1] / med[0] / 1e9, unit="GB/s", cores=1, kind=impl.kind,
+               sample="%d full steps (n=%d, %d sample positions) after 1 warm-up, median; %.1f ms/step"
+                      % (len(times), n, idx.size, med[0] * 1e3),
+               ms_per_step=med[0] * 1e3, prepare_ms=float(np.median([t[2] for t in times])) * 1e3,
+               compress_ms=float(np.median([t[3] for t in times])) * 1e3)
+    out.update(host_description())
+    return out
+
+
+def cpu_reduce_baseline(msgs_h, n, seconds):
+    """Config C5 on one host core: zero the dense vector, add the messages in rank order
+    (add_strategy), then residual += dense (the accumulate half of the broadcast-leg writeRemote)."""
+    from oracle.pyoracle import Oracle, ref_available
+    impl = Oracle(ref=True) if ref_available() else Oracle()
+    plain = Oracle()
+    dense = np.zeros(n, np.float32)
+    rests = np.zeros(n, np.float32)
+    red, app = [], []
+    t_end = time.perf_counter() + seconds
+    it = 0
+    while it < 2 or (time.perf_counter() < t_end and it < 50):
+        t0 = time.perf_counter()
+        dense[:] = 0
+        for m in msgs_h:
+            impl.ip_add(m, dense)
+        t1 = time.perf_counter()
+        plain.add_rests(rests, dense)
+        t2 = time.perf_counter()
+        if it > 0:
+            red.append(t1 - t0)
+            app.append(t2 - t1)
+        it += 1
+    return float(np.median(red)) * 1e3, float(np.median(app)) * 1e3, impl.kind, len(red)
 
 
 def main():
@@ -146,7 +205,34 @@ def main():
 
     extra = {"k_last_step": k, "density": k / n, "elements_per_s": n / (ms_per_step * 1e-3),
              "stage_kernel_ms": kern_ms, "rest_of_step_ms": ms_per_step - kern_ms,
-             "hbm_peak_fraction_step": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+             "hbm_peak_fraction_step": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+             "cache_state": "warm: consecutive steps, the residual's tail is still in the 256 MB memory-side cache"}
+
+    # the same step with a COLD residual: between two steps another kernel streams through 1 GiB
+    # (a training step's backward pass runs there), which evicts the 256 MB memory-side cache; the
+    # eviction itself is outside the events.  Two kinds: a kernel that only READS (the cache is left
+    # full of clean lines) and one that WRITES (left full of dirty lines, whose write-back then
+    # competes with the step).
+    evict = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)
+    cold_reps = max(5, min(args.steps, 20))
+    for key, what, fn in (("cold", "1 GiB read by another kernel between steps (memory-side cache evicted, clean)",
+                           lambda: evict.sum()),
+                          ("cold_after_writes", "1 GiB rewritten by another kernel between steps (cache evicted, dirty)",
+                           lambda: evict.add_(1.0))):
+        h.set_option("profile_stage", 1)
+        cold_step_ms = event_ms(torch, step, cold_reps, between=fn)
+        cold_stage = h.profile_read()
+        h.set_option("profile_stage", 0)
+        cold_kern_ms = float(np.mean(cold_stage))
+        extra[key] = {"what": what, "steps": cold_reps, "step_ms": cold_step_ms, "stage_kernel_ms": cold_kern_ms,
+                      "stage_kernel_GBps": kern_bytes / (cold_kern_ms * 1e-3) / 1e9,
+                      "stage_kernel_frac": kern_bytes / (cold_kern_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                      "step_GBps": step_bytes / (cold_step_ms * 1e-3) / 1e9,
+                      "hbm_peak_fraction_step": step_bytes / (cold_step_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        log("%s: step %.3f ms (%.1f%% of peak), streaming kernel %.3f ms (%.1f%% of peak)"
+            % (key, cold_step_ms, 100 * extra[key]["hbm_peak_fraction_step"], cold_kern_ms,
+               100 * extra[key]["stage_kernel_frac"]))
+    del evict
 
     if not args.no_extra:
         # what plain streaming reaches on this GPU, for scale: a device copy (8n bytes) and an
@@ -214,19 +300,40 @@ def main():
         msgs = [torch.from_numpy(mm).cuda() for mm in msgs_h]
         dense = torch.empty(c5n, device="cuda")
         red_bytes = 4 * c5n + 16 * len(msgs) * c5k
-        for mode, name in ((0, "reduce_ordered"), (1, "reduce_atomic")):
+        reduce = {"workload": W.C5["name"], "n": c5n, "ranks": len(msgs), "k_per_rank": c5k,
+                  "algorithmic_bytes": red_bytes, "peak": HBM_PEAK_GBPS, "unit": "GB/s"}
+        for mode, name in ((0, "ordered"), (1, "atomic")):
             for _ in range(2):
                 h.reduce(dense, msgs, accumulate=False, mode=mode)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                h.reduce(dense, msgs, accumulate=False, mode=mode)
-            torch.cuda.synchronize()
-            r_ms = (time.perf_counter() - t0) / reps * 1e3
-            extra[name + "_ms"] = r_ms
-            extra[name + "_GBps"] = red_bytes / (r_ms * 1e-3) / 1e9
-            log("%s %.3f ms (%.0f GB/s of 4n+16Rk)" % (name, r_ms, extra[name + "_GBps"]))
+            r_ms = event_ms(torch, lambda: h.reduce(dense, msgs, accumulate=False, mode=mode), reps)
+            reduce[name + "_ms"] = r_ms
+            reduce[name + "_GBps"] = red_bytes / (r_ms * 1e-3) / 1e9
+            reduce[name + "_frac"] = reduce[name + "_GBps"] / HBM_PEAK_GBPS
+            extra["reduce_" + name + "_ms"] = r_ms
+            extra["reduce_" + name + "_GBps"] = reduce[name + "_GBps"]
+            log("reduce %s %.3f ms (%.0f GB/s of 4n+16Rk, %.1f%% of peak)"
+                % (name, r_ms, reduce[name + "_GBps"], 100 * reduce[name + "_frac"]))
+        reduce["pairs_per_s"] = len(msgs) * c5k / (reduce["ordered_ms"] * 1e-3)
+        # residual apply (K4): rests += dense, 12 bytes per element
+        c5_rests = torch.zeros(c5n, device="cuda")
+        for _ in range(2):
+            h.add_vec(c5_rests, dense)
+        a_ms = event_ms(torch, lambda: h.add_vec(c5_rests, dense), reps)
+        apply_bytes = 12 * c5n
+        reduce["apply"] = {"algorithmic_bytes": apply_bytes, "ms": a_ms, "GBps": apply_bytes / (a_ms * 1e-3) / 1e9,
+                           "frac": apply_bytes / (a_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                           "elements_per_s": c5n / (a_ms * 1e-3)}
+        log("residual apply %.3f ms (%.0f GB/s of 12n, %.1f%% of peak)"
+            % (a_ms, reduce["apply"]["GBps"], 100 * reduce["apply"]["frac"]))
         h.synchronize()
+        if not args.no_cpu:
+            c_red, c_app, kind, cnt = cpu_reduce_baseline(msgs_h, c5n, min(args.cpu_seconds, 8.0))
+            reduce["cpu_baseline"] = {"cores": 1, "kind": kind, "sample": "%d full passes, median" % cnt,
+                                      "reduce_ms": c_red, "reduce_GBps": red_bytes / (c_red * 1e-3) / 1e9,
+                                      "apply_ms": c_app, "apply_GBps": apply_bytes / (c_app * 1e-3) / 1e9}
+            log("cpu baseline, reduce (%s, 1 core): %.1f ms (%.2f GB/s), apply %.1f ms (%.2f GB/s)"
+                % (kind, c_red, reduce["cpu_baseline"]["reduce_GBps"], c_app, reduce["cpu_baseline"]["apply_GBps"]))
+        extra["reduce"] = reduce
 
     cpu = None
     if not args.no_cpu:
@@ -252,8 +359,10 @@ def main():
         "config": {"workload": W.C4["name"], "n": n, "topK": float(topk), "sample_positions": m,
                    "threshold": "sampled ThresholdTopK over host-supplied positions", "input_checksum": W.checksum(g_h)},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(W.C4["name"], n), "kernel": "stage_kernel<float,0,4,%d>"
-                     % (args.items or 4), "algorithmic_bytes": kern_bytes, "avg_ms": kern_ms},
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(W.C4["name"], n),
+                     "traffic_source": "committed counter run profiles/stage_kernel_C4_100M_pmc.txt, not this run",
+                     "kernel": "stage_kernel<float,0,4,%d>" % (args.items or 4), "algorithmic_bytes": kern_bytes,
+                     "avg_ms": kern_ms, "cache_state": "warm (see extra.cold for the cold-residual figures)"},
         "cpu_baseline": cpu,
         "extra": extra,
     }

@@ -755,20 +755,41 @@ __global__ __launch_bounds__(kBlock) void zero_kernel(T* __restrict__ v, long lo
     for (long long i = nvec * VEC + (long long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) v[i] = (T)0;
 }
 
+// data[i] += rests[i].  A block owns kAddUnroll * kBlock consecutive 16-byte vectors; every load of a
+// thread is issued before the first add.  `rests` is read once and `data` rewritten once per call:
+// both go past the caches (nontemporal); the reads of `data` stay cacheable.
+constexpr int kAddUnroll = 4;
 template <typename T, int VEC>
 __global__ __launch_bounds__(kBlock) void add_vec_kernel(T* __restrict__ data, const T* __restrict__ rests,
                                                          long long n) {
-    const long long stride = (long long)gridDim.x * kBlock;
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
     const long long nvec = n / VEC;
-    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) {
-        Pack<T, VEC> a = reinterpret_cast<Pack<T, VEC>*>(data)[i];
-        const Pack<T, VEC> b = reinterpret_cast<const Pack<T, VEC>*>(rests)[i];
+    const long long first = (long long)blockIdx.x * (kBlock * kAddUnroll) + threadIdx.x;
+    if (VEC > 1 && first + (long long)(kAddUnroll - 1) * kBlock < nvec) {
+        vec_t a[kAddUnroll], b[kAddUnroll];
 #pragma unroll
-        for (int c = 0; c < VEC; ++c) a.x[c] = (T)(a.x[c] + b.x[c]);
-        reinterpret_cast<Pack<T, VEC>*>(data)[i] = a;
+        for (int q = 0; q < kAddUnroll; ++q) {
+            a[q] = reinterpret_cast<const vec_t*>(data)[first + q * kBlock];
+            b[q] = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(rests) + first + q * kBlock);
+        }
+#pragma unroll
+        for (int q = 0; q < kAddUnroll; ++q) {
+#pragma unroll
+            for (int c = 0; c < VEC; ++c) a[q][c] = (T)(a[q][c] + b[q][c]);
+            __builtin_nontemporal_store(a[q], reinterpret_cast<vec_t*>(data) + first + q * kBlock);
+        }
+    } else {
+        for (int q = 0; q < kAddUnroll; ++q) {
+            const long long v = first + (long long)q * kBlock;
+            if (v < nvec) {
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) data[v * VEC + c] = (T)(data[v * VEC + c] + rests[v * VEC + c]);
+            }
+        }
     }
-    for (long long i = nvec * VEC + (long long)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
-        data[i] = (T)(data[i] + rests[i]);
+    // elements behind the last whole vector
+    if (blockIdx.x == 0)
+        for (long long i = nvec * VEC + threadIdx.x; i < n; i += kBlock) data[i] = (T)(data[i] + rests[i]);
 }
 
 template <typename T>
@@ -842,12 +863,15 @@ template <typename T> int launch_add_vec(cx_handle h, T* data, const T* rests, i
     if (n < 0 || ((!data || !rests) && n > 0)) return fail(CX_ERR_INVALID, "add_vec: bad arguments");
     if (n == 0) return CX_OK;
     constexpr int kVec = 16 / (int)sizeof(T);
-    if (((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(rests)) & 15u) == 0)
-        hipLaunchKernelGGL((add_vec_kernel<T, kVec>), dim3(grid_for(n, 4 * kVec)), dim3(kBlock), 0, h->stream, data,
-                           rests, (long long)n);
-    else
-        hipLaunchKernelGGL((add_vec_kernel<T, 1>), dim3(grid_for(n, 4)), dim3(kBlock), 0, h->stream, data, rests,
-                           (long long)n);
+    if (((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(rests)) & 15u) == 0) {
+        const long long per_block = (long long)kBlock * kAddUnroll * kVec;
+        hipLaunchKernelGGL((add_vec_kernel<T, kVec>), dim3((unsigned)(((long long)n + per_block - 1) / per_block)),
+                           dim3(kBlock), 0, h->stream, data, rests, (long long)n);
+    } else {
+        const long long per_block = (long long)kBlock * kAddUnroll;
+        hipLaunchKernelGGL((add_vec_kernel<T, 1>), dim3((unsigned)(((long long)n + per_block - 1) / per_block)),
+                           dim3(kBlock), 0, h->stream, data, rests, (long long)n);
+    }
     CX_HIP(hipGetLastError());
     return CX_OK;
 }
