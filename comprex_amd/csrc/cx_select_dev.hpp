@@ -52,7 +52,11 @@ __device__ __forceinline__ void block_pick(const unsigned* hist, unsigned long l
     }
     __syncthreads();
     unsigned before = incl - local;
-    for (int w = 0; w < wave; ++w) before += (unsigned)s_sum[w];
+#pragma unroll
+    for (int w = 0; w < BLOCK / 64; ++w) {  // every wavefront reads all the sums at once, not one after the other
+        const unsigned sw = (unsigned)s_sum[w];
+        before += w < wave ? sw : 0u;
+    }
     if (want >= before && want - before < local) {
         unsigned acc = before;
 #pragma unroll

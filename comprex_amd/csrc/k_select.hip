@@ -215,120 +215,45 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
 }
 
 // ---- up to 2^18 keys: two launches --------------------------------------------------------
-// First launch: every block gathers KPT keys per thread, stores them to `keys` and counts their
-// top digit.  Second launch, one block: picks the top digit and finishes the remaining digits
-// alone, in LDS as soon as the keys still in play fit there.
+// First launch: every block gathers one key per thread, stores it to `keys` and counts its top
+// digit in LDS.  Second launch, one block: picks the digits alone, in LDS as soon as the keys
+// still in play fit there.
 //
 // One block has the instruction throughput and the memory bandwidth of one compute unit
 // (measured: about 50 GB/s, 7 us per 100 000 four-byte keys), so the second launch must not read
-// every key.  When the wanted key is near the top, each block of the first launch also passes on a
+// every key.  When the wanted key is near the top, each block of the first launch passes on a
 // SHORT LIST: its keys from the top digit of its own short_k-th largest key upwards (all its keys
-// when it has fewer), and the largest such digit over all blocks is recorded.  If the digit the
-// second launch picks is not below that, every key carrying it is in the short list and the
-// full key array is not needed; otherwise (large keys clustered in a few blocks, ties) the
-// second launch reads the key array, as it does when no short list was made.
+// when it has fewer), and the largest such digit over all blocks is recorded.  The list holds
+// EVERY key whose top digit is at least that one, so when more such keys exist than the wanted
+// rank, the answer is found from the list alone, and the first launch wrote nothing else: no block
+// adds its counts to the global histogram (those atomics queue up per digit: 2.5 to 6 us of
+// the first launch's 13.6 on 100 000 sampled positions).  Otherwise (large keys clustered in a few
+// blocks, ties, a list that overflowed) the second launch counts the key array itself.  Without a
+// short list the blocks merge their counts into the global histogram as the whole-vector passes do.
+//
+// One launch, with the block that finishes last doing the second launch's work, was measured
+// slower (30 us against 25): making the other blocks' keys visible inside one kernel takes a
+// device-wide release per block and an acquire in the last one, and on this GPU those write back
+// and invalidate the L2 of the block's XCD (0.5 to 1.2 us and 2.5 us; 30 us more with a fence in
+// every thread), which is what the launch boundary does anyway.
+#ifndef CX_FIRST_BLOCK
+#define CX_FIRST_BLOCK 1024
+#endif
+constexpr int kFirstBlock = CX_FIRST_BLOCK;  // threads per block of the first launch, one key each
 constexpr int kFinishBlock = 1024;
-constexpr int kListBytes = 32768;           // LDS list of the second launch
+constexpr int kListBytes = 49152;           // LDS list of the last block
 constexpr int kShortGlobalKeys = 1 << 16;   // capacity of the short list in device memory
 // Largest key count of this path.  Four keys per thread and 2^20 keys were measured too: no faster
-// than three histogram passes over the vector (63 vs 68 us at 2^20 keys), and the second
-// launch's worst case (no usable short list: it reads every key, up to three times) grows with
-// the key count.
+// than three histogram passes over the vector (63 vs 68 us at 2^20 keys), and the last block's
+// worst case (no usable short list: it reads every key, up to three times) grows with the key count.
 constexpr int kSmallSelect = 1 << 18;
-
-template <typename T, int SMODE, bool HAS_ADD, int KPT>
-__global__ __launch_bounds__(kFinishBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
-                                                              const int* __restrict__ idx, int m, int n, float stepsize,
-                                                              typename Elem<T>::key_t* __restrict__ keys,
-                                                              SelectState* __restrict__ st, int short_k,
-                                                              typename Elem<T>::key_t* __restrict__ short_keys,
-                                                              unsigned short_cap) {
-    using key_t = typename Elem<T>::key_t;
-    constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
-    constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
-    __shared__ unsigned lds_hist[kRadixBins];
-    __shared__ unsigned s_digit, s_base, s_wave[kFinishBlock / 64];
-    __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
-    // large blocks: every block ends with one global atomic per digit it has seen, and those
-    // queue up per address
-    for (int b = threadIdx.x; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
-    __syncthreads();
-    key_t mine[KPT];
-    bool have[KPT];
-    // the grid covers m; whole wavefronts take every step together (hist_add is a cross-lane operation)
-#pragma unroll
-    for (int q = 0; q < KPT; ++q) {
-        const long long i = ((long long)blockIdx.x * KPT + q) * kFinishBlock + threadIdx.x;
-        key_t k = 0;
-        have[q] = i < m;
-        if (have[q]) {
-            long long p;
-            bool ok = true;
-            if (SMODE == 0) {
-                p = i;
-            } else if (SMODE == 1) {
-                p = (long long)(int)__fmul_rn((float)(int)i, stepsize);  // (int)(i * stepsize), product in fp32
-                if (p > (long long)n - 1) p = (long long)n - 1;          // the reference would read out of bounds
-                if (p < 0) p = 0;
-            } else {
-                p = idx[i];
-                ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
-                if (!ok) p = 0;
-            }
-            T v = vec[p];
-            if (HAS_ADD) v = (T)(v + add[p]);
-            k = ok ? key_of(v) : (key_t)0;
-            keys[i] = k;
-        }
-        mine[q] = k;
-        hist_add(lds_hist, have[q], (unsigned)(k >> shift0) & kDigitMask);
-    }
-    merge_hist<kFinishBlock>(lds_hist, st);
-    if (short_k <= 0) return;
-
-    unsigned digit;
-    unsigned long long above;
-    block_pick<kFinishBlock>(lds_hist, (unsigned long long)(short_k - 1), s_sum, &s_digit, &s_above, digit, above);
-    unsigned outs = 0, cnt = 0;  // bit q: key q goes to the short list
-#pragma unroll
-    for (int q = 0; q < KPT; ++q) {
-        const bool out = have[q] && ((unsigned)(mine[q] >> shift0) & kDigitMask) >= digit;
-        outs |= (out ? 1u : 0u) << q;
-        cnt += out ? 1u : 0u;
-    }
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    unsigned incl = cnt;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const unsigned up = __shfl_up(incl, o, 64);
-        if (lane >= o) incl += up;
-    }
-    if (lane == 63) s_wave[wave] = incl;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned total = 0;
-        for (int w = 0; w < kFinishBlock / 64; ++w) total += s_wave[w];
-        s_base = atomicAdd(&st->short_count, total);
-        atomicMax(&st->short_digit, digit);
-    }
-    __syncthreads();
-    unsigned at = s_base + incl - cnt;
-    for (int w = 0; w < wave; ++w) at += s_wave[w];
-#pragma unroll
-    for (int q = 0; q < KPT; ++q)
-        if ((outs >> q) & 1u) {
-            if (at < short_cap) short_keys[at] = mine[q];  // an overflowing list is seen from its count
-            ++at;
-        }
-}
 
 // One block walks `count` keys that start on a 16-byte boundary and hands every key that still
 // matches the fixed digits to `hit`.  Written for one compute unit: sixteen 16-byte loads per lane
 // are in flight per round (a round trip to memory per round, not per key), and the test costs two
 // instructions per key.
 template <typename KEY, typename HIT>
-__device__ __forceinline__ void scan_matching(const KEY* __restrict__ src, unsigned count, KEY prefix, KEY mask,
-                                              HIT hit) {
+__device__ __forceinline__ void scan_matching(const KEY* src, unsigned count, KEY prefix, KEY mask, HIT hit) {
     constexpr int KV = 16 / (int)sizeof(KEY);  // keys per 16-byte load
     constexpr int kLoads = 16;
     const int t = threadIdx.x;
@@ -343,7 +268,7 @@ __device__ __forceinline__ void scan_matching(const KEY* __restrict__ src, unsig
                 kk[q] = kv[v];
             } else {
 #pragma unroll
-                for (int c = 0; c < KV; ++c) kk[q].x[c] = ~prefix;  // never matches
+                for (int c = 0; c < KV; ++c) kk[q].x[c] = (KEY)0;
             }
         }
 #pragma unroll
@@ -351,7 +276,7 @@ __device__ __forceinline__ void scan_matching(const KEY* __restrict__ src, unsig
             bool any = false;
 #pragma unroll
             for (int c = 0; c < KV; ++c) any |= (kk[q].x[c] & mask) == prefix;
-            if (any) {
+            if (any && v0 + q * kFinishBlock + t < nfull) {  // (an empty mask matches the padding too)
 #pragma unroll
                 for (int c = 0; c < KV; ++c)
                     if ((kk[q].x[c] & mask) == prefix) hit(kk[q].x[c]);
@@ -364,6 +289,93 @@ __device__ __forceinline__ void scan_matching(const KEY* __restrict__ src, unsig
     }
 }
 
+template <typename T, int SMODE, bool HAS_ADD>
+__global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                              const int* __restrict__ idx, int m, int n, float stepsize,
+                                                              typename Elem<T>::key_t* __restrict__ keys,
+                                                              SelectState* __restrict__ st, int short_k,
+                                                              typename Elem<T>::key_t* __restrict__ short_keys,
+                                                              unsigned short_cap) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
+    constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
+    __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit, s_base, s_wave[kFirstBlock / 64];
+    __shared__ unsigned long long s_above, s_sum[kFirstBlock / 64];
+    const int t = threadIdx.x;
+    const bool short_on = short_k > 0;
+
+    // ---- every block: gather, count, pass on
+    for (int b = t; b < kRadixBins; b += kFirstBlock) lds_hist[b] = 0u;
+    __syncthreads();
+    // the grid covers m; whole wavefronts take every step together (hist_add is a cross-lane operation)
+    const long long i = (long long)blockIdx.x * kFirstBlock + t;
+    key_t mine = 0;
+    const bool have = i < m;
+    if (have) {
+        long long p;
+        bool ok = true;
+        if (SMODE == 0) {
+            p = i;
+        } else if (SMODE == 1) {
+            p = (long long)(int)__fmul_rn((float)(int)i, stepsize);  // (int)(i * stepsize), product in fp32
+            if (p > (long long)n - 1) p = (long long)n - 1;          // the reference would read out of bounds
+            if (p < 0) p = 0;
+        } else {
+            p = idx[i];
+            ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+            if (!ok) p = 0;
+        }
+        T v = vec[p];
+        if (HAS_ADD) v = (T)(v + add[p]);
+        mine = ok ? key_of(v) : (key_t)0;
+        keys[i] = mine;
+    }
+    hist_add(lds_hist, have, (unsigned)(mine >> shift0) & kDigitMask);
+    if (!short_on) {
+        merge_hist<kFirstBlock>(lds_hist, st);
+    } else {
+        __syncthreads();
+        unsigned digit;
+        unsigned long long above;
+        block_pick<kFirstBlock>(lds_hist, (unsigned long long)(short_k - 1), s_sum, &s_digit, &s_above, digit, above);
+        const bool out = have && ((unsigned)(mine >> shift0) & kDigitMask) >= digit;
+        const unsigned long long outs = __ballot(out);
+        const int lane = t & 63, wave = t >> 6;
+        if (lane == 0) s_wave[wave] = (unsigned)__popcll(outs);
+        __syncthreads();
+        if (t == 0) {
+            unsigned total = 0;
+            for (int w = 0; w < kFirstBlock / 64; ++w) total += s_wave[w];
+            s_base = atomicAdd(&st->short_count, total);
+            atomicMax(&st->short_digit, digit);
+        }
+        __syncthreads();
+        unsigned at = s_base + (unsigned)__popcll(outs & ((1ull << lane) - 1ull));
+        for (int w = 0; w < wave; ++w) at += s_wave[w];
+        if (out && at < short_cap) short_keys[at] = mine;  // an overflowing list is seen from its count
+    }
+
+}
+
+// Bitwise AND and OR over the wavefront.
+template <typename KEY> __device__ __forceinline__ void wave_and_or(KEY& a, KEY& o) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        a &= (KEY)__shfl_xor(a, off, 64);
+        o |= (KEY)__shfl_xor(o, off, 64);
+    }
+}
+
+// The second launch.  A short list that fits LDS is moved there in one round trip to memory,
+// keeping only the keys from the digit on from which the list is complete.  Those keys share
+// their leading bits (they are the largest few percent): the digits are taken from the first bit
+// in which they differ, so that ONE histogram spreads them over the bins, and as soon as at most
+// kDirect keys are left the wanted one is found by counting, for each, the keys above it.
+// Everything else (no short list, a list too long for LDS, a rank the list does not reach) walks
+// the fixed digits from the top, as the whole-vector passes do.
+constexpr int kDirect = 256;
+
 template <typename T>
 __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typename Elem<T>::key_t* __restrict__ keys,
                                                                      int m, SelectState* __restrict__ st,
@@ -373,47 +385,127 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
                                                                      unsigned short_cap) {
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
-    constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
     constexpr int kListKeys = kListBytes / (int)sizeof(key_t);
-    __shared__ unsigned lds_hist[kRadixBins];
+    constexpr int shift0 = kKeyBits - kRadixBits;
+    constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
+    constexpr key_t kAllBits = (key_t)(~(key_t)0) >> (8 * (int)sizeof(key_t) - kKeyBits);
+    static_assert(kDirect * sizeof(key_t) <= kRadixBins * sizeof(unsigned), "the candidates reuse the histogram");
+    __shared__ __align__(8) unsigned lds_hist[kRadixBins];
     __shared__ key_t s_list[kListKeys];
+    __shared__ key_t s_and, s_or, s_answer;
     __shared__ unsigned s_digit, s_fill;
     __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
     const int t = threadIdx.x;
+    const int lane = t & 63;
 
-    // top digit: counted by the first launch into the global histogram
-    for (int b = t; b < kRadixBins; b += kFinishBlock) {
-        lds_hist[b] = st->hist[b];
-        st->hist[b] = 0u;  // leave it clean for the next run
-    }
     // what the first launch's blocks passed on
     const unsigned short_count = short_on ? st->short_count : 0u;
     const unsigned short_digit = short_on ? st->short_digit : 0u;
+    for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
+    if (t == 0) {
+        s_fill = 0u;
+        s_and = kAllBits;
+        s_or = (key_t)0;
+    }
     __syncthreads();
     if (short_on && t == 0) {  // clean for the next run
         st->short_count = 0u;
         st->short_digit = 0u;
     }
     key_t prefix = 0, mask = 0;
+    int lo = kKeyBits;  // the bits below this one are still open
     // where the keys still in play are read from: the key array, the short list, or (listed) LDS
     const key_t* src = keys;
     unsigned src_n = (unsigned)m;
-    bool listed = false;
+    bool listed = false, counted = false;
     unsigned list_n = 0;
-    for (int p = 0; p < kPasses; ++p) {
-        int shift = kKeyBits - kRadixBits * (p + 1);
-        int bits = kRadixBits;
-        if (shift < 0) {
-            bits += shift;
-            shift = 0;
+    if (short_on && short_count <= (unsigned)kListKeys && short_count <= short_cap) {
+        constexpr int kPer = kListKeys / kFinishBlock;
+        key_t kk[kPer];
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            const unsigned j = (unsigned)(q * kFinishBlock + t);
+            kk[q] = j < short_count ? short_keys[j] : (key_t)0;
         }
+        key_t all_and = kAllBits, all_or = (key_t)0;
+#pragma unroll
+        for (int q = 0; q < kPer; ++q) {
+            if ((unsigned)(q * kFinishBlock) < short_count) {  // the same for the whole block
+                const unsigned j = (unsigned)(q * kFinishBlock + t);
+                const bool in = j < short_count && ((unsigned)(kk[q] >> shift0) & kDigitMask) >= short_digit;
+                const unsigned long long ins = __ballot(in);
+                unsigned base = 0;
+                if (lane == 0 && ins) base = atomicAdd(&s_fill, (unsigned)__popcll(ins));
+                base = __shfl(base, 0, 64);
+                if (in) {
+                    s_list[base + (unsigned)__popcll(ins & ((1ull << lane) - 1ull))] = kk[q];
+                    all_and &= kk[q];
+                    all_or |= kk[q];
+                }
+            }
+        }
+        wave_and_or<key_t>(all_and, all_or);
+        if (lane == 0) {
+            atomicAnd(&s_and, all_and);
+            atomicOr(&s_or, all_or);
+        }
+        __syncthreads();
+        const unsigned complete = s_fill;
+        if (rank < (unsigned long long)complete) {  // the wanted key is one of these
+            counted = true;
+            listed = true;
+            list_n = complete;
+            const key_t differ = s_and ^ s_or;
+            lo = differ ? 64 - __clzll((unsigned long long)differ) : 0;
+            const key_t open_bits = lo >= 8 * (int)sizeof(key_t) ? (key_t)~(key_t)0 : (key_t)(((key_t)1 << lo) - 1);
+            mask = kAllBits & ~open_bits;
+            prefix = s_and & mask;
+        }
+    } else if (short_on && short_count <= short_cap) {
+        // top digits of the short list, from the digit on from which the list is complete
+        unsigned seen = 0;
+        scan_matching<key_t>(short_keys, short_count, (key_t)0, (key_t)0, [&](key_t k1) {
+            const unsigned d = (unsigned)(k1 >> shift0) & kDigitMask;
+            if (d >= short_digit) {
+                atomicAdd(&lds_hist[d], 1u);
+                ++seen;
+            }
+        });
+        if (seen) atomicAdd(&s_fill, seen);
+        __syncthreads();
+        if (rank < (unsigned long long)s_fill) {
+            counted = true;
+            src = short_keys;
+            src_n = short_count;
+        }
+    }
+    __syncthreads();
+    bool hist_ready = counted && !listed;
+    if (!counted) {
+        if (short_on) {  // nobody merged counts: count the top digit of every key
+            for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
+            __syncthreads();
+            scan_matching<key_t>(keys, (unsigned)m, (key_t)0, (key_t)0,
+                                 [&](key_t k1) { atomicAdd(&lds_hist[(unsigned)(k1 >> shift0) & kDigitMask], 1u); });
+        } else {
+            for (int b = t; b < kRadixBins; b += kFinishBlock) {
+                lds_hist[b] = st->hist[b];
+                st->hist[b] = 0u;  // leave it clean for the next run
+            }
+        }
+        hist_ready = true;
+        __syncthreads();
+    }
+    while (lo > 0) {
+        const int bits = lo < kRadixBits ? lo : kRadixBits;
+        const int shift = lo - bits;
         const unsigned digit_mask = (1u << bits) - 1u;
-        if (p > 0) {
+        if (!hist_ready) {
             for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
             __syncthreads();
             if (listed) {
-                for (unsigned i = t; i < list_n; i += kFinishBlock) {
-                    const key_t k1 = s_list[i];
+                for (unsigned j = t; j < list_n; j += kFinishBlock) {
+                    const key_t k1 = s_list[j];
                     if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 }
             } else {
@@ -423,6 +515,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             }
             __syncthreads();
         }
+        hist_ready = false;
         unsigned digit;
         unsigned long long above;
         block_pick<kFinishBlock>(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
@@ -430,11 +523,9 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         prefix |= (key_t)digit << shift;
         mask |= (key_t)((1ull << bits) - 1ull) << shift;
         rank -= above;
-        if (p == 0 && short_on && short_count <= short_cap && digit >= short_digit) {
-            src = short_keys;  // holds every key with the picked top digit
-            src_n = short_count;
-        }
-        if (!listed && p + 1 < kPasses && in_digit <= (unsigned)kListKeys) {
+        lo = shift;
+        if (lo == 0) break;
+        if (!listed && in_digit <= (unsigned)kListKeys) {
             // collect the keys still in play; their order does not matter
             if (t == 0) s_fill = 0u;
             __syncthreads();
@@ -444,6 +535,35 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             listed = true;
         }
         __syncthreads();
+        if (listed && in_digit <= (unsigned)kDirect && in_digit > 0u) {
+            // few keys left: the wanted one has at most `rank` keys above it and more than `rank`
+            // keys at or above it
+            key_t* cand = reinterpret_cast<key_t*>(lds_hist);
+            if (t == 0) {
+                s_fill = 0u;
+                s_answer = prefix;  // (a rank beyond the keys leaves the open bits zero, as the digits would)
+            }
+            __syncthreads();
+            for (unsigned j = t; j < list_n; j += kFinishBlock) {
+                const key_t k1 = s_list[j];
+                if ((k1 & mask) == prefix) cand[atomicAdd(&s_fill, 1u)] = k1;
+            }
+            __syncthreads();
+            const unsigned c = s_fill;  // == in_digit
+            if ((unsigned)t < c) {
+                const key_t me = cand[t];
+                unsigned gt = 0, ge = 0;
+                for (unsigned j = 0; j < c; ++j) {
+                    const key_t x = cand[j];
+                    gt += x > me ? 1u : 0u;
+                    ge += x >= me ? 1u : 0u;
+                }
+                if ((unsigned long long)gt <= rank && rank < (unsigned long long)ge) s_answer = me;
+            }
+            __syncthreads();
+            prefix = s_answer;
+            lo = 0;
+        }
     }
     if (t == 0) {
         T v = value_of(prefix, T());
@@ -613,8 +733,7 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
         }
         key_t* keys = static_cast<key_t*>(h->sel_keys);
         key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) + h->sel_keys_bytes);
-        constexpr int kpt = 1;  // keys per thread of the first launch
-        const int per_block = kFinishBlock * kpt;
+        const int per_block = kFirstBlock;
         const int blocks = (m + per_block - 1) / per_block;
         // short list: worth it when the wanted rank is near the top, so that a block's share of the
         // keys above it (plus 8 sigma) is a small part of the block, and the shares fit the list
@@ -622,19 +741,19 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
         const double share = (double)(rank + 1) / (double)blocks;
         int short_k = (int)(share + 8.0 * std::sqrt(share) + 8.0);
         if (!h->select_short_list || m < 8192 || short_k > per_block / 4 ||
-            (double)blocks * (short_k + 16.0 * kpt) > (double)short_cap)
+            (double)blocks * (short_k + 16.0) > (double)short_cap)
             short_k = 0;
-#define CX_FIRST(SM, HA, KPT)                                                                                           \
-    hipLaunchKernelGGL((select_first_kernel<T, SM, HA, KPT>), dim3(blocks), dim3(kFinishBlock), 0, h->stream, vec,      \
-                       add_vec, d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
-#define CX_FIRST_MODE(HA, KPT)                                   \
-    do {                                                         \
-        if (sample_mode == kSampleFull) CX_FIRST(0, HA, KPT);    \
-        else if (sample_mode == kSampleStrided) CX_FIRST(1, HA, KPT); \
-        else CX_FIRST(2, HA, KPT);                               \
+#define CX_FIRST(SM, HA)                                                                                             \
+    hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kFirstBlock), 0, h->stream, vec, add_vec, \
+                       d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
+#define CX_FIRST_MODE(HA)                                      \
+    do {                                                       \
+        if (sample_mode == kSampleFull) CX_FIRST(0, HA);       \
+        else if (sample_mode == kSampleStrided) CX_FIRST(1, HA); \
+        else CX_FIRST(2, HA);                                  \
     } while (0)
-        if (add_vec) CX_FIRST_MODE(true, kpt);
-        else CX_FIRST_MODE(false, kpt);
+        if (add_vec) CX_FIRST_MODE(true);
+        else CX_FIRST_MODE(false);
 #undef CX_FIRST_MODE
 #undef CX_FIRST
         hipLaunchKernelGGL(select_finish_kernel<T>, dim3(1), dim3(kFinishBlock), 0, h->stream, keys, m, h->sel, rank,

@@ -369,7 +369,10 @@ def test_sampled_threshold_short_list_and_inputs_that_defeat_it(dev, oracle, dty
     """The two-launch select hands its second launch a short list of each block's top keys and
     falls back on the full key array when the list cannot hold the answer: large values
     clustered in a few blocks' share of the samples, all-equal keys (list overflows), sample sets
-    too small or ranks too deep for the list.  Same threshold as the checker with the list on and off."""
+    too small or ranks too deep for the list.  The second launch takes its digits from the first bit in
+    which the listed keys differ and ranks the last few keys by counting: inputs with few distinct
+    magnitudes (ties) and with keys that differ in their first bit.  Same threshold as the checker
+    with the list on and off."""
     rng = np.random.default_rng(31)
     n = 3_000_000
     if dtype == np.int32:
@@ -382,8 +385,16 @@ def test_sampled_threshold_short_list_and_inputs_that_defeat_it(dev, oracle, dty
     clustered[: n // 40] = spread[: n // 40]            # every large value sits at the front
     equal = np.full(n, 7, dtype)
     zero = np.zeros(n, dtype)
+    # few distinct magnitudes: the keys left for the final count are full of ties
+    quantized = (spread // 100_000 * 100_000 if dtype == np.int32 else np.round(spread * 2) / 2).astype(dtype)
+    # the largest keys are the largest there are (-INT_MAX: the magnitude of INT_MIN is no int, and
+    # the reference's abs() of it is undefined)
+    extreme = spread.copy()
+    extreme[:: 37] = -np.iinfo(np.int32).max if dtype == np.int32 else np.finfo(dtype).max
+    extreme[5 :: 41] = np.iinfo(np.int32).max if dtype == np.int32 else np.finfo(dtype).tiny
     try:
-        for name, v, a in [("spread", spread, add), ("clustered", clustered, zero), ("equal", equal, zero)]:
+        for name, v, a in [("spread", spread, add), ("clustered", clustered, zero), ("equal", equal, zero),
+                           ("quantized", quantized, zero), ("extreme", extreme, zero)]:
             gv, ga = _gpu(v), _gpu(a)
             for m, topk in [(100_000, 0.01), (65_536, 0.0133), (8_192, 0.01), (200_000, 0.002), (100_000, 0.2),
                             (262_144, 0.01), (5_000, 0.01), (262_145, 0.01), (700_001, 0.003)]:
