@@ -286,6 +286,84 @@ def test_optimizer_trains_over_simulated_ranks(schedule):
         assert np.isfinite(last) and last < 0.7 * first, (schedule, rank, first, last)
 
 
+@pytest.mark.parametrize("schedule", ["comprex_alltoone", "comprex_ring", "comprex_bigring"])
+def test_optimizer_over_ranks_adds_up_to_the_closed_form(schedule):
+    """Four ranks, five steps, integer gradients, momentum 1/2, learning rate 1, no clipping, no weight
+    decay: every momentum term is a dyadic rational, so every sum below is exact in fp32 whatever
+    the compressor holds back and in whatever order it is added.  What the compressed allreduce
+    delays it delivers with the flush, so after the steps plus one flush (applied like a step)
+
+        w = w0 - (1/R) * sum over ranks q and steps s of m[q][s],   m[q][s] = m[q][s-1] / 2 + g[q][s]
+
+    wherever the schedule delivers everything: on every rank for the big ring, on the chief for
+    all-to-one (its broadcast is compressed without a flush, src/allreduce.tpp:196-239), and for
+    the ring on the segment a rank finishes itself (the others arrive thresholded, without a
+    residual, src/allreduce.tpp:441-457).  The expectation is computed here in float64 from the
+    gradients alone; nothing of the library or the checker takes part in it."""
+    import threading
+    from comprex_amd import pygpi
+    from comprex_amd.optimizer import ComprexOptimizer
+    R, dim, steps = 4, 6002, 5
+    rng = np.random.default_rng(77)
+    grads = rng.integers(-8, 9, (R, steps, dim)).astype(np.float64)
+    grads[:, :, ::7] *= 16                       # a heavy tail, so that the top-k has something to prefer
+    w0 = rng.integers(-100, 101, dim).astype(np.float64)
+    m = np.zeros((R, dim))
+    total = np.zeros(dim)
+    for s in range(steps):
+        m = 0.5 * m + grads[:, s]
+        total += m.sum(axis=0)
+    want = (w0 - total / R).astype(np.float32)
+    assert (want.astype(np.float64) == w0 - total / R).all()   # the expectation itself is exact in fp32
+    env = pygpi.GaspiEnvironment()
+    env.set_rank(0, R)
+    env.set_blocking(True, 60.0)
+    got, held_back, errors = {}, {}, []
+
+    def rank_program(rank):
+        try:
+            env.set_rank(rank, R)
+            w = torch.nn.Parameter(torch.from_numpy(w0.astype(np.float32)).cuda())
+            opt = ComprexOptimizer([w], env, learning_rate=1.0, momentum=0.5, compression_ratio=0.05,
+                                   allreduce_type=schedule, size_factor=3.0, pre_clipnorm=1e30)
+            for s in range(steps):
+                env.barrier()
+                w.grad = torch.from_numpy(grads[rank, s].astype(np.float32)).cuda()
+                opt.step()
+            env.barrier()
+            # what is still held back arrives with the flush; it is applied like a step
+            opt.blob.zero_()
+            opt.allreduce.flush(opt.blob)
+            held_back[rank] = int(torch.count_nonzero(opt.blob))
+            with torch.no_grad():
+                w.sub_(opt.blob / R)
+            got[rank] = w.detach().cpu().numpy()
+            env.barrier()
+        except Exception as e:  # noqa: BLE001
+            errors.append((rank, repr(e)))
+
+    threads = [threading.Thread(target=rank_program, args=(r,)) for r in range(R)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(180)
+    assert not errors, errors
+    if schedule == "comprex_bigring":
+        for r in range(R):
+            assert (got[r] == want).all(), (schedule, r)
+        assert all(held_back[r] > 0 for r in range(R))       # the compressor did hold something back
+    elif schedule == "comprex_alltoone":
+        assert (got[0] == want).all()
+        assert held_back[0] > 0
+    else:
+        sizes = [dim // R + (1 if c < dim % R else 0) for c in range(R)]
+        starts = np.concatenate([[0], np.cumsum(sizes)])
+        for r in range(R):
+            c = (r + 1) % R
+            assert (got[r][starts[c]:starts[c + 1]] == want[starts[c]:starts[c + 1]]).all(), (schedule, r)
+        assert all(held_back[r] > 0 for r in range(R))
+
+
 def test_sampled_step_can_be_captured_in_a_hip_graph():
     """threshold (left on the device) + compress enqueue kernels only, so a caller may capture them.
     Two steps (one in each walking direction) are captured and replayed three times, with eager
