@@ -323,3 +323,31 @@ def parse_message(msg, dtype):
     rec = np.dtype([("i", np.int32), ("v", dt)], align=False)
     body = np.frombuffer(msg[8:8 + int(k) * rec.itemsize].tobytes(), dtype=rec)
     return int(n), int(k), body["i"].copy(), body["v"].copy()
+
+
+def reorder_bound(msgs, dtype, n, base=None):
+    """How far two floating-point sums of the same contributions can lie apart when only the ORDER
+    of the additions differs (rank order against whatever order atomics take), per element.
+
+    Element i receives c_i contributions v_1..v_c (plus base[i] when given), summed from a start
+    that is one of the terms (or from zero, whose first addition is exact): c_i - 1 (with a base:
+    c_i) rounded additions.  Each ordering's result differs from the exact sum by at most
+    gamma_m * sum|v|, gamma_m = m*u / (1 - m*u), m the number of rounded additions, u = eps/2 the unit
+    roundoff (Higham, Accuracy and Stability of Numerical Algorithms, section 4.2); two orderings
+    differ by at most twice that.  An element with a single contribution and no base has bound 0:
+    both paths must give the same bits there.  Computed in float64 from the messages alone."""
+    dt = np.dtype(dtype)
+    u = float(np.finfo(dt).eps) / 2.0
+    mass = np.zeros(n, np.float64)
+    count = np.zeros(n, np.int64)
+    for m in msgs:
+        _, _, idx, val = parse_message(np.asarray(m), dt)
+        np.add.at(mass, idx, np.abs(val.astype(np.float64)))
+        np.add.at(count, idx, 1)
+    rounded = np.maximum(count - 1, 0)
+    if base is not None:
+        mass += np.abs(np.asarray(base, np.float64))
+        rounded = count
+    gamma = rounded * u / (1.0 - rounded * u)
+    # the bound itself is evaluated in float64: one part in 2^40 of slack covers its own rounding
+    return 2.0 * gamma * mass * (1.0 + 2.0 ** -40)

@@ -512,3 +512,46 @@ def test_fast_comprex_conserves_what_it_is_given(oracle, codec, dtype):
         copied = a.halves[a.half_bytes * ((a.st[1] + 1) % 2):][:a.st[0]].copy()
     add(a.flush_rests(), got_a)
     assert np.array_equal(got_a, total) and not a.rests.any()
+
+
+def test_reorder_bound_holds_for_other_orders_and_vanishes_for_single_contributions():
+    """The bound the atomic reduce is held to, tried on the CPU: the same contributions summed in
+    fp32 in rank order, in reverse order and in two shuffled orders stay within it of each other,
+    ill-conditioned (cancelling) elements included; where one message contributes it is zero."""
+    from oracle.pyoracle import reorder_bound
+    rng = np.random.default_rng(3)
+    n, ranks, k = 5000, 8, 1500
+    msgs, pairs = [], []
+    for r in range(ranks):
+        idx = np.sort(rng.choice(n, k, replace=False)).astype(np.int32)
+        val = (rng.standard_normal(k) * 10.0 ** rng.integers(-3, 4, k)).astype(np.float32)
+        if r % 2:  # cancellation against the previous message wherever both hit
+            prev_i, prev_v = pairs[-1]
+            both = np.isin(idx, prev_i)
+            val[both] = -prev_v[np.searchsorted(prev_i, idx[both])] * np.float32(1.0 + 2.0 ** -12)
+        rec = np.zeros(k, np.dtype([("i", np.int32), ("v", np.float32)]))
+        rec["i"], rec["v"] = idx, val
+        msgs.append(np.concatenate([np.array([n, k], np.int32).view(np.uint8), rec.view(np.uint8)]))
+        pairs.append((idx, val))
+    bound = reorder_bound(msgs, np.float32, n)
+
+    def summed(order, base=None):
+        out = np.zeros(n, np.float32) if base is None else base.copy()
+        for r in order:
+            out[pairs[r][0]] += pairs[r][1]
+        return out
+    ref = summed(range(ranks))
+    worst = 0.0
+    for order in (range(ranks - 1, -1, -1), rng.permutation(ranks), rng.permutation(ranks)):
+        diff = np.abs(summed(order).astype(np.float64) - ref.astype(np.float64))
+        assert (diff <= bound).all()
+        worst = max(worst, float((diff / np.maximum(bound, 1e-300)).max()))
+    assert worst > 0.05          # not a vacuous bound: some element comes within a factor 20 of it
+    count = np.zeros(n, np.int64)
+    for i, _ in pairs:
+        count[i] += 1
+    assert ((bound == 0.0) == (count <= 1)).all()
+    base = rng.standard_normal(n).astype(np.float32)
+    bound_b = reorder_bound(msgs, np.float32, n, base)
+    assert (np.abs(summed(range(ranks - 1, -1, -1), base).astype(np.float64) - summed(range(ranks), base)) <= bound_b).all()
+    assert ((bound_b == 0.0) == (count == 0)).all()
