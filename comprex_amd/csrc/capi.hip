@@ -144,6 +144,18 @@ int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_b
 
 }  // namespace
 
+namespace {
+template <typename T> int reserve_impl(cx_handle h, int n, unsigned paths) {
+    int rc = CX_OK;
+    if (rc == CX_OK && (paths & CX_RESERVE_COMPRESS)) rc = reserve_compact<T>(h, n);
+    if (rc == CX_OK && (paths & CX_RESERVE_THRESHOLD)) rc = reserve_select<T>(h, n);
+    if (rc == CX_OK && (paths & CX_RESERVE_REDUCE)) rc = reserve_reduce<T>(h, n);
+    if (rc == CX_OK && (paths & CX_RESERVE_RLE)) rc = reserve_rle<T>(h, n);
+    return rc;
+}
+}  // namespace
+
+
 extern "C" {
 
 const char* cx_last_error(void) { return last_error().c_str(); }
@@ -386,6 +398,12 @@ int cx_ip_compress_noalloc(cx_handle h, cx_dtype dt, void* out_msg, long long ou
 }
 
 long long cx_noalloc_max_elements(void) { return noalloc_max_elements(); }
+
+int cx_reserve(cx_handle h, cx_dtype dt, int n, unsigned paths) {
+    if (!h || n < 0) return fail(CX_ERR_INVALID, "cx_reserve: null handle or negative size");
+    if (paths == 0u || (paths & ~(unsigned)CX_RESERVE_ALL)) return fail(CX_ERR_INVALID, "cx_reserve: unknown path bits %#x", paths);
+    CX_DISPATCH(dt, reserve_impl<T>(h, n, paths));
+}
 
 int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
                         int n, float topK, void* d_thr_out, int* d_size_prefix, int* h_bytes) {

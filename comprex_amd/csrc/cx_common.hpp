@@ -141,6 +141,11 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
                    const T* thr_host, const T* d_thr, int* d_size_prefix, bool no_alloc = false);
 // allocation-free variant: this device's copy of the static scratch array, and its size limit
 int locate_static_scratch(unsigned** out);
+// Pre-size a module's scratch for vectors of up to n elements of T, so that later calls find it large enough.
+template <typename T> int reserve_compact(cx_handle h, int n);
+template <typename T> int reserve_select(cx_handle h, int n);
+template <typename T> int reserve_reduce(cx_handle h, int n);
+template <typename T> int reserve_rle(cx_handle h, int n);
 long long noalloc_max_elements();
 
 template <typename T>

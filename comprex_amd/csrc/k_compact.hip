@@ -481,6 +481,16 @@ int ensure_scratch(cx_handle h, size_t ntiles, size_t staging_words) {
     return CX_OK;
 }
 
+// Largest scratch any tile shape needs for n elements of T: the smallest tile (2 vectors per lane)
+// has the most tiles; the slots hold an eighth of the elements whatever the shape.
+template <typename T> void scratch_need(long long n, size_t* ntiles, size_t* staging_words) {
+    constexpr int kVec = 16 / (int)sizeof(T);
+    constexpr int PW = Elem<T>::pair_words;
+    constexpr long long kSmallestTile = 64ll * kVec * 2, kLargestTile = 64ll * kVec * 8;
+    *ntiles = (size_t)((n + kSmallestTile - 1) / kSmallestTile);
+    *staging_words = (size_t)((n + kLargestTile - 1) / kLargestTile) * (size_t)(kLargestTile / 8) * PW;
+}
+
 template <typename T, int MODE, int VEC, int ITEMS>
 int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
                long long cap_pairs, int* size_prefix, DeviceStatus* status, bool no_alloc) {
@@ -797,6 +807,15 @@ CX_INSTANTIATE_FUSED(double)
 CX_INSTANTIATE_FUSED(int)
 #undef CX_INSTANTIATE_FUSED
 
+template <typename T> int reserve_compact(cx_handle h, int n) {
+    size_t ntiles, words;
+    scratch_need<T>(n, &ntiles, &words);
+    if (ntiles < (size_t)kFilterBlocks * kWavesPerBlock) ntiles = (size_t)kFilterBlocks * kWavesPerBlock;  // launch_filter
+    return ensure_scratch(h, ntiles, words);
+}
+template int reserve_compact<float>(cx_handle, int);
+template int reserve_compact<double>(cx_handle, int);
+template int reserve_compact<int>(cx_handle, int);
 template int launch_compact<float>(cx_handle, void*, long long, const float*, float*, int, const float*, const float*, int*, bool);
 template int launch_compact<double>(cx_handle, void*, long long, const double*, double*, int, const double*, const double*, int*, bool);
 template int launch_compact<int>(cx_handle, void*, long long, const int*, int*, int, const int*, const int*, int*, bool);

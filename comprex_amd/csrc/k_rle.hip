@@ -451,6 +451,17 @@ int launch_rle_decode(cx_handle h, T* out, int out_n, const void* msg, int add, 
     return CX_OK;
 }
 
+template <typename T> int reserve_rle(cx_handle h, int n) {
+    int rc = ensure_bytes(h, &h->rle_pairs, &h->rle_pairs_bytes, 8 + (size_t)n * 4 * Elem<T>::pair_words);
+    if (rc != CX_OK) return rc;
+    rc = ensure_bytes(h, reinterpret_cast<void**>(&h->rle_scan), &h->rle_scan_bytes, (size_t)kConvBlocks * sizeof(unsigned));
+    if (rc != CX_OK) return rc;
+    return reserve_compact<T>(h, n);  // the pairs are made by the compaction
+}
+template int reserve_rle<float>(cx_handle, int);
+template int reserve_rle<double>(cx_handle, int);
+template int reserve_rle<int>(cx_handle, int);
+
 #define CX_INSTANTIATE_RLE(T)                                                                                   \
     template int launch_rle_compress<T>(cx_handle, void*, long long, const T*, T*, int, const T*, const T*, int*, int*); \
     template int launch_rle_decode<T>(cx_handle, T*, int, const void*, int, int*);

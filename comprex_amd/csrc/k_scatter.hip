@@ -704,12 +704,8 @@ int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n
     return CX_OK;
 }
 
-template <typename T>
-int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
-    if (out_n == 0) return CX_OK;
-    constexpr int kReduceTile = ReduceTile<T>::value;
-    const unsigned ntiles = (unsigned)(((long long)out_n + kReduceTile - 1) / kReduceTile);
-    const size_t need = (size_t)kMaxMsgs * (ntiles + 1);
+// first pair of each message in each dense tile, for the tiled reduce
+int ensure_bounds(cx_handle h, size_t need) {
     if (need > h->reduce_bounds_cap) {
         CX_HIP(hipStreamSynchronize(h->stream));
         if (h->reduce_bounds) CX_HIP(hipFree(h->reduce_bounds));
@@ -718,6 +714,16 @@ int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_
         CX_HIP(hipMalloc(reinterpret_cast<void**>(&h->reduce_bounds), need * sizeof(unsigned)));
         h->reduce_bounds_cap = need;
     }
+    return CX_OK;
+}
+
+template <typename T>
+int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
+    if (out_n == 0) return CX_OK;
+    constexpr int kReduceTile = ReduceTile<T>::value;
+    const unsigned ntiles = (unsigned)(((long long)out_n + kReduceTile - 1) / kReduceTile);
+    int rc_bounds = ensure_bounds(h, (size_t)kMaxMsgs * (ntiles + 1));
+    if (rc_bounds != CX_OK) return rc_bounds;
     for (int first = 0; first < n_msgs || first == 0; first += kMaxMsgs) {
         MsgList list;
         const int cnt = n_msgs - first < kMaxMsgs ? n_msgs - first : kMaxMsgs;
@@ -941,6 +947,15 @@ int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n
     }
     return CX_OK;
 }
+
+template <typename T> int reserve_reduce(cx_handle h, int n) {
+    constexpr int kReduceTile = ReduceTile<T>::value;
+    const size_t ntiles = (size_t)(((long long)n + kReduceTile - 1) / kReduceTile);
+    return ensure_bounds(h, (size_t)kMaxMsgs * (ntiles + 1));
+}
+template int reserve_reduce<float>(cx_handle, int);
+template int reserve_reduce<double>(cx_handle, int);
+template int reserve_reduce<int>(cx_handle, int);
 
 #define CX_INSTANTIATE(T)                                                                         \
     template int launch_zero<T>(cx_handle, T*, int);                                              \

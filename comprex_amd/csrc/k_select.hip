@@ -714,6 +714,38 @@ template <typename T> void pass_digits(int p, int* shift, int* bits, int* last) 
 }  // namespace
 
 // The key of descending rank `rank` among the m keys described by (vec, add_vec, d_idx, mode).
+// key array of the two-launch select (2 MB), then its short list
+int ensure_select_keys(cx_handle h) {
+    const size_t want_bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
+    if (h->sel_keys_bytes < want_bytes) {
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->sel_keys) CX_HIP(hipFree(h->sel_keys));
+        h->sel_keys = nullptr;
+        h->sel_keys_bytes = 0;
+        CX_HIP(hipMalloc(&h->sel_keys, want_bytes + (size_t)kShortGlobalKeys * sizeof(unsigned long long)));
+        h->sel_keys_bytes = want_bytes;
+    }
+    return CX_OK;
+}
+
+// candidate buffer of the one-pass exact selections
+int ensure_candidates(cx_handle h, size_t need) {
+    if (need > h->cand_bytes) {
+        CX_HIP(hipStreamSynchronize(h->stream));
+        if (h->cand) CX_HIP(hipFree(h->cand));
+        h->cand = nullptr;
+        h->cand_bytes = 0;
+        CX_HIP(hipMalloc(&h->cand, need + 256));
+        h->cand_bytes = need;
+    }
+    return CX_OK;
+}
+
+// candidates kept for a vector of m elements: a sixteenth of it, at least 4 Mi
+inline size_t candidate_capacity(long long m) {
+    return (size_t)m / 16 > ((size_t)1 << 22) ? (size_t)m / 16 : ((size_t)1 << 22);
+}
+
 template <typename T>
 int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
                 float stepsize, unsigned long long rank, int plus_one, T* d_thr_out) {
@@ -721,16 +753,8 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
     using key_t = typename Elem<T>::key_t;
 
     if (m <= kSmallSelect) {
-        // key array (2 MB), then the short list
-        const size_t want_bytes = (size_t)kSmallSelect * sizeof(unsigned long long);
-        if (h->sel_keys_bytes < want_bytes) {
-            CX_HIP(hipStreamSynchronize(h->stream));
-            if (h->sel_keys) CX_HIP(hipFree(h->sel_keys));
-            h->sel_keys = nullptr;
-            h->sel_keys_bytes = 0;
-            CX_HIP(hipMalloc(&h->sel_keys, want_bytes + (size_t)kShortGlobalKeys * sizeof(unsigned long long)));
-            h->sel_keys_bytes = want_bytes;
-        }
+        int rc_keys = ensure_select_keys(h);
+        if (rc_keys != CX_OK) return rc_keys;
         key_t* keys = static_cast<key_t*>(h->sel_keys);
         key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) + h->sel_keys_bytes);
         const int per_block = kFirstBlock;
@@ -798,15 +822,9 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;
     if (m < (1 << 23) || sample_rank >= (unsigned long long)kSample / 16 || !vec_ok) return CX_OK;
 
-    const size_t cap = (size_t)m / 16 > ((size_t)1 << 22) ? (size_t)m / 16 : ((size_t)1 << 22);
-    if (cap * sizeof(key_t) > h->cand_bytes) {
-        CX_HIP(hipStreamSynchronize(h->stream));
-        if (h->cand) CX_HIP(hipFree(h->cand));
-        h->cand = nullptr;
-        h->cand_bytes = 0;
-        CX_HIP(hipMalloc(&h->cand, cap * sizeof(key_t) + 256));
-        h->cand_bytes = cap * sizeof(key_t);
-    }
+    const size_t cap = candidate_capacity(m);
+    int rc_cand = ensure_candidates(h, cap * sizeof(key_t));
+    if (rc_cand != CX_OK) return rc_cand;
     // 1. lower bound from the sample, left in the second half of the threshold slot
     T* d_bound = reinterpret_cast<T*>(static_cast<char*>(h->d_thr) + 64);
     unsigned* d_count = reinterpret_cast<unsigned*>(static_cast<char*>(h->d_thr) + 128);
@@ -875,22 +893,15 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
         return launch_compact<T>(h, out_msg, out_capacity, data, update, n, nullptr, d_thr_out, d_size_prefix);
     }
 
-    const size_t cap = (size_t)n / 16 > ((size_t)1 << 22) ? (size_t)n / 16 : ((size_t)1 << 22);
-    const size_t need = 8 + cap * PW * 4;
-    if (need > h->cand_bytes) {
-        CX_HIP(hipStreamSynchronize(h->stream));
-        if (h->cand) CX_HIP(hipFree(h->cand));
-        h->cand = nullptr;
-        h->cand_bytes = 0;
-        CX_HIP(hipMalloc(&h->cand, need + 256));
-        h->cand_bytes = need;
-    }
+    const size_t cap = candidate_capacity(n);
+    int rc = ensure_candidates(h, 8 + cap * PW * 4);
+    if (rc != CX_OK) return rc;
     unsigned* cand_words = static_cast<unsigned*>(h->cand);
     T* d_bound = reinterpret_cast<T*>(static_cast<char*>(h->d_thr) + 64);
     unsigned* d_result = reinterpret_cast<unsigned*>(static_cast<char*>(h->d_thr) + 128);
 
     // 1. lower bound
-    int rc = select_rank<T>(h, update, data, n, nullptr, kSample, kSampleStrided, (float)n / (float)kSample, sample_rank,
+    rc = select_rank<T>(h, update, data, n, nullptr, kSample, kSampleStrided, (float)n / (float)kSample, sample_rank,
                             0, d_bound);
     if (rc != CX_OK) return rc;
     // 2. accumulate + candidates
@@ -942,6 +953,17 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
     return select_rank<T>(h, vec, add_vec, n, d_idx, m, sample_mode, stepsize, rank, plus_one, d_thr_out);
 }
 
+template <typename T> int reserve_select(cx_handle h, int n) {
+    int rc = ensure_select_keys(h);
+    if (rc != CX_OK) return rc;
+    if (n < (1 << 23)) return CX_OK;  // shorter vectors never take the one-pass selections
+    const size_t cap = candidate_capacity(n);
+    const size_t as_keys = cap * sizeof(typename Elem<T>::key_t), as_pairs = 8 + cap * Elem<T>::pair_words * 4;
+    return ensure_candidates(h, as_keys > as_pairs ? as_keys : as_pairs);
+}
+template int reserve_select<float>(cx_handle, int);
+template int reserve_select<double>(cx_handle, int);
+template int reserve_select<int>(cx_handle, int);
 template int launch_topk_threshold<float>(cx_handle, const float*, const float*, int, const int*, int, int, float, float, float*);
 template int launch_topk_threshold<double>(cx_handle, const double*, const double*, int, const int*, int, int, float, float, double*);
 template int launch_topk_threshold<int>(cx_handle, const int*, const int*, int, const int*, int, int, float, float, int*);

@@ -56,6 +56,14 @@ class Handle:
         except Exception:
             pass
 
+    RESERVE_COMPRESS, RESERVE_THRESHOLD, RESERVE_REDUCE, RESERVE_RLE, RESERVE_ALL = 1, 2, 4, 8, 15
+
+    def reserve(self, n, dtype, paths=7):
+        """Sizes the handle's scratch for vectors of up to n elements of `dtype` so that later calls
+        on the named paths (an OR of the RESERVE_* bits; default: all but the run-length codec) never
+        allocate (cx_reserve)."""
+        check(self.lib.cx_reserve(self._h, _DT[dtype], int(n), int(paths)))
+
     def set_option(self, key, value):
         check(self.lib.cx_set_option(self._h, key.encode(), int(value)))
 

@@ -146,10 +146,25 @@ public:
         return *this;
     }
 
-    void setCompressor(const Compressor<VarTYPE>& c) { this->compressor.reset(c.clone()); }
-    void setCompressor(const Compressor<VarTYPE>* c) { this->compressor.reset(c->clone()); }
-    void setThreshold(const ThresholdFunction<VarTYPE>& t) { this->threshold.reset(t.clone()); }
-    void setThreshold(const ThresholdFunction<VarTYPE>* t) { this->threshold.reset(t->clone()); }
+    void setCompressor(const Compressor<VarTYPE>& c) { setCompressor(&c); }
+    void setCompressor(const Compressor<VarTYPE>* c) {
+        this->compressor.reset(c->clone());
+        reserve_scratch();
+    }
+    void setThreshold(const ThresholdFunction<VarTYPE>& t) { setThreshold(&t); }
+    void setThreshold(const ThresholdFunction<VarTYPE>* t) {
+        this->threshold.reset(t->clone());
+        reserve_scratch();
+    }
+
+    // The GPU scratch of the clones this object owns, sized for this object's vectors when the
+    // clones are made: the exchange calls then never allocate.  Without a GPU (objects built only to
+    // be configured) nothing is reserved.
+    void reserve_scratch() {
+        if (size <= 0 || cx_device_count() < 1) return;
+        threshold->reserve(size);
+        compressor->reserve(size, threshold->whole_vector_topk(size, nullptr));
+    }
 
     void print_rests() {
         std::vector<VarTYPE> r = getRests();

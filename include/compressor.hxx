@@ -57,6 +57,14 @@ public:
     // Not in the reference: bytes of the largest message a vector of n elements can produce.
     virtual long long max_message_bytes(int n) const = 0;
 
+    // Not in the reference: sizes this compressor's GPU scratch for vectors of up to n elements, so
+    // that the exchange itself never allocates (the reference takes its memory in the constructors
+    // too, src/comprEx.tpp:40-60).  `whole_vector_topk`: the one-pass exact top-k will be used.
+    virtual void reserve(int n, bool whole_vector_topk) {
+        cxx::check(cx_reserve(handle_.get(), cxx::dtype_of<VarTYPE>::value, n,
+                              reserve_paths() | (whole_vector_topk ? (unsigned)CX_RESERVE_THRESHOLD : 0u)));
+    }
+
     // Not in the reference: waits for this compressor's GPU work and returns (and forgets) the first
     // error a kernel recorded since the last call, CX_OK if none.  A message cut short for lack of
     // room (CX_ERR_CAPACITY) is valid as far as it goes; what it could not hold stayed in the
@@ -95,6 +103,7 @@ protected:
         }
     }
 
+    virtual unsigned reserve_paths() const { return CX_RESERVE_COMPRESS | CX_RESERVE_REDUCE; }
     cxx::Handle handle_;
     cxx::DeviceBuffer stage_msg_, stage_a_, stage_b_;
 };
@@ -221,6 +230,10 @@ public:
     // n values, n + 1 run lengths at most
     virtual long long max_message_bytes(int n) const { return 16 + (long long)n * (long long)sizeof(VarTYPE) + 4ll * ((long long)n + 1); }
 
+protected:
+    virtual unsigned reserve_paths() const { return CX_RESERVE_RLE | CX_RESERVE_REDUCE; }
+public:
+
     virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
                                 const VarTYPE* d_threshold, VarTYPE threshold, int* d_size_prefix, bool wait) {
         if (!d_data && !d_update) throw std::runtime_error("Compression needs a valid input vector!");
@@ -307,6 +320,7 @@ public:
     CompressorNone(const CompressorNone<VarTYPE>& other) : Compressor<VarTYPE>(other) {}
     virtual Compressor<VarTYPE>* clone() const { return new CompressorNone<VarTYPE>(*this); }
     virtual long long max_message_bytes(int n) const { return 4 + (long long)n * (long long)sizeof(VarTYPE); }
+    virtual void reserve(int, bool) {}  // copies and adds only: no scratch
 
     virtual int compress_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
                                 const VarTYPE*, VarTYPE, int* d_size_prefix, bool) {

@@ -67,6 +67,22 @@ int cx_device_alloc(void** out, size_t bytes);
 int cx_device_free(void* p);
 int cx_copy(cx_handle h, void* dst, const void* src, size_t bytes);
 
+/* The handle's scratch buffers grow on demand, which makes a call that finds them too small wait for
+ * the stream and allocate.  cx_reserve sizes them ahead of time for vectors of up to n elements of
+ * type `dt`, for the paths named in `paths` (an OR of the bits below), so that none of those calls
+ * allocates afterwards.  It plays the part of the constructors' allocations in the reference
+ * (ComprEx's restsVector and buffers, src/comprEx.tpp:40-60): memory is taken when the object is set
+ * up, not in the exchange.  CX_RESERVE_RLE takes 8 + n * (4 + sizeof(T)) bytes (the pairs its
+ * encoder starts from); the others take about n/2 bytes or less. */
+enum {
+    CX_RESERVE_COMPRESS = 1,   /* cx_ip_compress, the compaction of cx_ip_compress_topk */
+    CX_RESERVE_THRESHOLD = 2,  /* cx_topk_threshold*, the candidate list of cx_ip_compress_topk */
+    CX_RESERVE_REDUCE = 4,     /* cx_ip_decompress, cx_ip_add, cx_ip_reduce on vectors of n elements */
+    CX_RESERVE_RLE = 8,        /* cx_rle_compress */
+    CX_RESERVE_ALL = 15
+};
+int cx_reserve(cx_handle h, cx_dtype dt, int n, unsigned paths);
+
 /* No counterpart in the reference, whose transports take a host-side byte count
  * (initTransferPart(sizeBytes, offset), src/comprEx.tpp:442): copies *d_bytes bytes (a device
  * int32, e.g. the size prefix a compressor wrote; clamped to [0, capacity]) from src to dst, device

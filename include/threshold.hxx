@@ -51,6 +51,8 @@ public:
 
     // Device address of the current threshold, or nullptr when only the host value exists.
     virtual const VarTYPE* device_threshold() { return nullptr; }
+    // Not in the reference: sizes the GPU scratch of this threshold for vectors of up to n elements.
+    virtual void reserve(int n) {}
 
     // Not in the reference.  True when prepare_with on n elements would apply the top-k rule to
     // every element (no sub-sampling); the fraction is returned.  ComprEx then computes threshold
@@ -166,6 +168,10 @@ public:
 
     virtual const VarTYPE* device_threshold() {
         return on_device_ ? static_cast<const VarTYPE*>(cx_threshold_slot(this->handle_.get())) : nullptr;
+    }
+
+    virtual void reserve(int n) {
+        cxx::check(cx_reserve(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, n, CX_RESERVE_THRESHOLD));
     }
 
     // n < subsamples is the reference's test for using the whole vector (src/threshold.hxx:224-231)

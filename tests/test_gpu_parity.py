@@ -46,6 +46,46 @@ def _msgbuf(n, dtype, extra=0):
     return torch.zeros(message_capacity(n, NP2T[dtype]) + extra, dtype=torch.uint8, device="cuda")
 
 
+def test_reserve_takes_the_scratch_up_front(oracle):
+    """cx_reserve sizes a handle's scratch once; the calls that follow, on vectors up to the reserved
+    length, leave the device's free memory where it was (they would otherwise grow their buffers on
+    first use) and give the checker's results."""
+    from comprex_amd.device import Handle, message_capacity
+    n = 9_000_000          # above 2^23: the one-pass exact top-k and its candidate list are in play
+    rng = np.random.default_rng(12)
+    g_h = rng.laplace(size=n).astype(np.float32)
+    g, r = _gpu(g_h), torch.zeros(n, device="cuda")
+    msg = torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+    rle = torch.zeros(16 + 8 * n + 8, dtype=torch.uint8, device="cuda")
+    idx = _gpu(np.sort(rng.integers(0, n, 50_000)).astype(np.int32))
+    dense = torch.zeros(n, device="cuda")
+    h = Handle()
+    try:
+        with pytest.raises(RuntimeError):
+            h.reserve(n, torch.float32, 0)
+        with pytest.raises(RuntimeError):
+            h.reserve(n, torch.float32, 32)
+        h.reserve(n, torch.float32, Handle.RESERVE_ALL)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        thr = h.topk_threshold_indexed(r, g, idx, np.float32(0.01))
+        assert thr == oracle.topk_prepare_indexed(np.zeros(n, np.float32), g_h, idx.cpu().numpy(), np.float32(0.01))
+        nbytes = h.compress(msg, g, r)
+        want_r = np.zeros(n, np.float32)
+        want = oracle.ip_compress(g_h, want_r, np.float32(thr))
+        assert msg[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        h.decompress(dense, msg)
+        h.reduce(dense, [msg, msg], accumulate=False, mode=0)
+        h.reduce(dense, [msg, msg], accumulate=True, mode=0)
+        h.compress_topk(msg, g, r, np.float32(0.001))
+        assert h.get_option("fused_topk_taken") == 1   # the one-pass route, whose candidate list was reserved
+        h.rle_compress(rle, g, r, thr=np.float32(thr))
+        h.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+    finally:
+        h.close()
+
+
 # --------------------------------------------------------------------------- K2
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("mode", ["fused", "update", "data"])
