@@ -138,6 +138,13 @@ int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_b
     if (rc != CX_OK || !h_bytes) return rc;
     CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
     rc = collect_status(h);
+    if (rc == CX_ERR_INDEX) {
+        // the fast path wants ascending indices; the reference takes any order (src/compressor.hxx:613-633):
+        // once more, pair after pair.  An index outside the vector is reported again.
+        rc = launch_sequential<T>(h, static_cast<T*>(out), out_n, msg, 0);
+        if (rc != CX_OK) return rc;
+        rc = collect_status(h);
+    }
     *h_bytes = 8 + h->h_pinned[9] * 4 * Elem<T>::pair_words;
     return rc;
 }

@@ -171,6 +171,8 @@ template <typename T> int launch_rle_decode(cx_handle h, T* out, int out_n, cons
 
 template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg);
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);
+// the reference's loop, pair after pair: any index order, indices repeated anywhere (slow)
+template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, const void* msg, int add);
 template <typename T>
 int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode);
 int launch_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity);

@@ -78,6 +78,55 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(T* __restrict__ out, in
     if (bad) atomicCAS(&status->code, 0, (int)CX_ERR_INDEX);
 }
 
+struct MsgHeaders {
+    static constexpr int kMax = 16;
+    const unsigned* msg[kMax];
+};
+
+// The reference's loop for ANY message (src/compressor.hxx:613-658): pairs in the order they are
+// stored, indices in any order, repeated anywhere.  One wavefront takes 64 pairs at a time; the
+// chunks follow each other, and a chunk in which two pairs share an index is applied lane by lane.
+// Slow (tens of ns per pair): the fallback for messages the sorted paths refuse.
+template <typename T, int OP>
+__global__ __launch_bounds__(64) void sequential_kernel(T* out, int out_n,
+                                                       const unsigned* __restrict__ msg, DeviceStatus* status) {
+    constexpr int PW = Elem<T>::pair_words;
+    const int n_msg = (int)msg[0];
+    const long long k = (long long)(int)msg[1];
+    if (n_msg > out_n) {
+        if (threadIdx.x == 0) atomicCAS(&status->code, 0, (int)CX_ERR_MSG_TOO_LARGE);
+        return;
+    }
+    const unsigned* pairs = msg + 2;
+    const int lane = threadIdx.x;
+    bool bad = false;
+    for (long long j0 = 0; j0 < k; j0 += 64) {
+        const long long j = j0 + lane;
+        const bool live = j < k;
+        const int idx = live ? (int)pairs[PW * j] : -1;
+        const bool ok = live && (unsigned)idx < (unsigned)out_n;
+        bad |= live && !ok;
+        const T v = ok ? load_value<T>(pairs + PW * j + 1) : (T)0;
+        bool shared = false;  // an earlier lane of this chunk has the same index
+        for (int l = 0; l < 63; ++l) {
+            const int other = __shfl(idx, l, 64);
+            shared |= ok && l < lane && other == idx;
+        }
+        if (__ballot(shared) == 0ull) {
+            if (ok) out[idx] = OP == 0 ? v : (T)(out[idx] + v);
+        } else {
+            for (int l = 0; l < 64; ++l) {
+                if (l == lane && ok) out[idx] = OP == 0 ? v : (T)(out[idx] + v);
+                __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+                __builtin_amdgcn_s_waitcnt(0);  // the store has left before the next lane reads the element
+            }
+        }
+        // the next chunk may touch the same elements: this one's stores come first
+        __threadfence_block();
+    }
+    if (bad) atomicCAS(&status->code, 0, (int)CX_ERR_INDEX);
+}
+
 // ---- tiled, rank-ordered reduce ------------------------------------------------------------
 // out (+)= sum of up to kMaxMsgs index-sorted messages, applied in the order given, with the
 // dense vector written exactly once:
@@ -674,9 +723,28 @@ __global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out,
     if (bad) atomicCAS(&status->code, 0, (int)CX_ERR_INDEX);
 }
 
+// An empty output vector: nothing to write, but a message made for a longer vector is still an
+// error (the reference throws, src/compressor.hxx:620-624,645-647).
+__global__ void header_check_kernel(MsgHeaders list, int n_msgs, DeviceStatus* status) {
+    for (int r = threadIdx.x; r < n_msgs; r += blockDim.x)
+        if ((int)list.msg[r][0] > 0) atomicCAS(&status->code, 0, (int)CX_ERR_MSG_TOO_LARGE);
+}
+
+int check_headers(cx_handle h, const void* const* msgs, int n_msgs) {
+    for (int first = 0; first < n_msgs; first += MsgHeaders::kMax) {
+        MsgHeaders list;
+        const int cnt = n_msgs - first < MsgHeaders::kMax ? n_msgs - first : MsgHeaders::kMax;
+        for (int r = 0; r < MsgHeaders::kMax; ++r)
+            list.msg[r] = r < cnt ? static_cast<const unsigned*>(msgs[first + r]) : nullptr;
+        hipLaunchKernelGGL(header_check_kernel, dim3(1), dim3(64), 0, h->stream, list, cnt, h->d_status);
+    }
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
 template <typename T>
 int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
-    if (out_n == 0) return CX_OK;
+    if (out_n == 0) return check_headers(h, msgs, n_msgs);
     constexpr int kTile = MergeTile<T>::value;
     const unsigned ntiles = (unsigned)(((long long)out_n + kTile - 1) / kTile);
     // persistent blocks: a few per compute unit, each with a contiguous run of tiles
@@ -719,7 +787,7 @@ int ensure_bounds(cx_handle h, size_t need) {
 
 template <typename T>
 int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
-    if (out_n == 0) return CX_OK;
+    if (out_n == 0) return check_headers(h, msgs, n_msgs);
     constexpr int kReduceTile = ReduceTile<T>::value;
     const unsigned ntiles = (unsigned)(((long long)out_n + kReduceTile - 1) / kReduceTile);
     int rc_bounds = ensure_bounds(h, (size_t)kMaxMsgs * (ntiles + 1));
@@ -894,8 +962,24 @@ int launch_threshold_apply(cx_handle h, T* high, T* low, const T* in, int n, con
     return CX_OK;
 }
 
+template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, const void* msg, int add) {
+    if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "decompress: bad arguments");
+    if (!add) {
+        int rc = launch_zero<T>(h, out, out_n);
+        if (rc != CX_OK) return rc;
+        hipLaunchKernelGGL((sequential_kernel<T, 0>), dim3(1), dim3(64), 0, h->stream, out, out_n,
+                           static_cast<const unsigned*>(msg), h->d_status);
+    } else {
+        hipLaunchKernelGGL((sequential_kernel<T, 1>), dim3(1), dim3(64), 0, h->stream, out, out_n,
+                           static_cast<const unsigned*>(msg), h->d_status);
+    }
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic) {
-    if (!out || !msg || out_n < 0) return fail(CX_ERR_INVALID, "add: bad arguments");
+    if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "add: bad arguments");
+    if (out_n == 0) return check_headers(h, &msg, 1);
     const unsigned* words = static_cast<const unsigned*>(msg);
     const unsigned grid = grid_for(out_n, 1);  // k <= n <= out_n for any message that passes the size check
     if (atomic)
@@ -909,7 +993,8 @@ template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void*
 }
 
 template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg) {
-    if (!out || !msg || out_n < 0) return fail(CX_ERR_INVALID, "decompress: bad arguments");
+    if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "decompress: bad arguments");
+    if (out_n == 0) return check_headers(h, &msg, 1);
     // one message: short-lived blocks, one per tile, reach the vector's write rate; the pipelined
     // kernel (reduce_variant 3 forces it) pays off from two messages on
     if (h->reduce_variant == 0 || h->reduce_variant == 2) return launch_tiled<T>(h, out, out_n, &msg, 1, 0, 0);
@@ -924,7 +1009,8 @@ template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, cons
 
 template <typename T>
 int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode) {
-    if (!out || out_n < 0 || n_msgs < 0 || (n_msgs > 0 && !msgs)) return fail(CX_ERR_INVALID, "reduce: bad arguments");
+    if ((!out && out_n > 0) || out_n < 0 || n_msgs < 0 || (n_msgs > 0 && !msgs)) return fail(CX_ERR_INVALID, "reduce: bad arguments");
+    if (out_n == 0) return check_headers(h, msgs, n_msgs);
     if (mode == 0 && h->reduce_variant == 3) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
     if (mode == 0 && h->reduce_variant == 0 && !accumulate && n_msgs > 1) {
         // measured on 64 Mi fp32 elements with 1 %-dense messages: writing the vector from zeros, the
@@ -962,6 +1048,7 @@ template int reserve_reduce<int>(cx_handle, int);
     template int launch_add_vec<T>(cx_handle, T*, const T*, int);                                 \
     template int launch_threshold_apply<T>(cx_handle, T*, T*, const T*, int, const T*, const T*); \
     template int launch_add<T>(cx_handle, T*, int, const void*, int);                             \
+    template int launch_sequential<T>(cx_handle, T*, int, const void*, int);                      \
     template int launch_decompress<T>(cx_handle, T*, int, const void*);                           \
     template int launch_reduce<T>(cx_handle, T*, int, const void* const*, int, int, int);
 CX_INSTANTIATE(float)

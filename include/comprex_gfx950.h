@@ -209,7 +209,13 @@ int cx_rle_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg);
 
 /* CompressorIndexPairs<T>::decompression_strategy (src/compressor.hxx:613-638): zero
  * all out_n elements, then out[index] = value.  A message whose n exceeds out_n leaves
- * `out` zeroed and records CX_ERR_MSG_TOO_LARGE.  h_bytes as above (bytes consumed). */
+ * `out` zeroed and records CX_ERR_MSG_TOO_LARGE.  h_bytes as above (bytes consumed).
+ * Index order: the compressors of this library and of the reference emit ascending indices, and
+ * the fast path requires them (an index below its predecessor records CX_ERR_INDEX).  The
+ * reference's decoder takes any order, repeats anywhere, last value wins: with h_bytes != NULL
+ * (the call waits anyway) such a message is decoded once more, pair after pair, with exactly that
+ * result; with h_bytes == NULL the error stands.  Indices outside [0, out_n) are CX_ERR_INDEX
+ * either way (the reference writes out of bounds). */
 int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes);
 
 /* CompressorIndexPairs<T>::add_strategy (src/compressor.hxx:640-658): out[index] += value
@@ -221,8 +227,12 @@ int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, i
 /* The chief's reduce loop of Comprex_AllToOneAllreduce::apply (src/allreduce.tpp:183-189):
  * out (+)= sum over messages in the order given.  `msgs` is a HOST array of n_msgs device
  * pointers.  accumulate == 0 starts from zeros (every message is added, the first one to
- * 0), != 0 adds into `out`.  mode 0 = rank-ordered, bit-exact; mode 1 =
- * floating-point atomics (order of additions unspecified). */
+ * 0), != 0 adds into `out`.  mode 0 = rank-ordered, bit-exact, needs every message's indices
+ * ascending (CX_ERR_INDEX otherwise; option reduce_variant = 1 only needs equal indices to be
+ * neighbours); mode 1 = one launch of floating-point atomics per message, in the order given:
+ * the additions to an element are reordered only among pairs of ONE message that share its
+ * index.  An empty `out` (out_n == 0) writes nothing and still refuses messages made for a
+ * longer vector (CX_ERR_MSG_TOO_LARGE). */
 int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* const* msgs, int n_msgs,
                  int accumulate, int mode);
 

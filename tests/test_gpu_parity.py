@@ -700,6 +700,60 @@ def test_tiled_reduce_reports_unsorted_message(dev):
     assert e.value.code == _lib.CX_ERR_INDEX
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decompress_takes_any_index_order_when_it_reports_back(dev, oracle, dtype):
+    """The reference's decoder walks the pairs as stored (src/compressor.hxx:613-633): any index order,
+    an index repeated anywhere, the last value wins.  The fast path wants ascending indices; a
+    decompress that reports its byte count to the host repeats such a message pair after pair.
+    Expected values: the checker, which is that loop.  Out-of-range indices stay errors, and an
+    empty output vector still refuses a message made for a longer one."""
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rng = np.random.default_rng(41)
+    n, k = 50_000, 9_001
+    idx = rng.integers(0, n, k).astype(np.int32)                  # unsorted, with repeats far apart
+    idx[100:110] = idx[5000]                                        # and a run of repeats inside one chunk
+    val = _rand(rng, k, dtype)
+    rec = np.dtype([("i", np.int32), ("v", dtype)])
+    body = np.empty(k, rec)
+    body["i"], body["v"] = idx, val
+    msg = np.concatenate([np.array([n, k], np.int32).view(np.uint8), body.view(np.uint8)])
+    want = np.full(n, 9, dtype)
+    oracle.ip_decompress(msg, want)
+    by_hand = np.zeros(n, dtype)
+    for i, v in zip(idx, val):
+        by_hand[i] = v
+    assert want.tobytes() == by_hand.tobytes()
+    g = torch.full((n,), 7, dtype=NP2T[dtype], device="cuda")
+    assert dev.decompress(g, _gpu(msg)) == msg.size
+    assert g.cpu().numpy().tobytes() == want.tobytes()
+    # without the report the message is refused, not half applied silently
+    dev.decompress(g, _gpu(msg), sync=False)
+    with pytest.raises(ComprexError) as e:
+        dev.synchronize()
+    assert e.value.code == _lib.CX_ERR_INDEX
+    # an index outside the vector is an error on both paths
+    body["i"][17] = n + 3
+    bad = np.concatenate([np.array([n, k], np.int32).view(np.uint8), body.view(np.uint8)])
+    with pytest.raises(ComprexError) as e:
+        dev.decompress(g, _gpu(bad))
+    assert e.value.code == _lib.CX_ERR_INDEX
+    # empty output vector
+    empty = torch.zeros(0, dtype=NP2T[dtype], device="cuda")
+    for variant in (0, 3):
+        dev.set_option("reduce_variant", variant)
+        try:
+            dev.reduce(empty, [_gpu(msg)], accumulate=False, mode=0)
+            with pytest.raises(ComprexError) as e:
+                dev.synchronize()
+            assert e.value.code == _lib.CX_ERR_MSG_TOO_LARGE
+            none = np.array([0, 0], np.int32).view(np.uint8)
+            dev.reduce(empty, [_gpu(none)], accumulate=False, mode=0)
+            dev.synchronize()
+        finally:
+            dev.set_option("reduce_variant", 0)
+
+
 # --------------------------------------------------------------------------- residual maintenance
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_zero_addvec_apply(dev, oracle, dtype):
