@@ -63,7 +63,7 @@ struct SelectState {
     unsigned long long rank;       // descending rank still to find among matching keys
     unsigned int hist[kRadixBins]; // digit histogram of the current pass
     unsigned int short_count;      // two-launch select: keys in the short list; zero between runs
-    unsigned int short_digit;      // ... and the largest digit a block cut its share at
+    unsigned int short_digit;      // ... and the largest cut of a block: the leading two digits of its short_k-th key
     // chained passes (no pick launch in between): one histogram per pass, all zero between runs,
     // and the state entering each pass
     unsigned int pass_hist[kMaxRadixPasses][kRadixBins];

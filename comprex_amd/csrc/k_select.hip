@@ -225,11 +225,11 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
 // SHORT LIST: its keys from the top digit of its own short_k-th largest key upwards (all its keys
 // when it has fewer), and the largest such digit over all blocks is recorded.  The list holds
 // EVERY key whose top digit is at least that one, so when more such keys exist than the wanted
-// rank, the answer is found from the list alone, and the first launch wrote nothing else: no block
-// adds its counts to the global histogram (those atomics queue up per digit: 2.5 to 6 us of
-// the first launch's 13.6 on 100 000 sampled positions).  Otherwise (large keys clustered in a few
-// blocks, ties, a list that overflowed) the second launch counts the key array itself.  Without a
-// short list the blocks merge their counts into the global histogram as the whole-vector passes do.
+// rank, the answer is found from the list alone.  Otherwise (large keys clustered in a few
+// blocks, ties, keys that all share their top digit so that the list overflows) the second launch
+// starts from the top-digit counts of ALL keys, which every block of the first launch adds to the
+// global histogram either way (leaving that out made the first launch 0.7 us faster and this
+// case 60 us slower: the one block would have to count every key again), and reads the key array.
 //
 // One launch, with the block that finishes last doing the second launch's work, was measured
 // slower (30 us against 25): making the other blocks' keys visible inside one kernel takes a
@@ -298,6 +298,7 @@ __global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __re
                                                               unsigned short_cap) {
     using key_t = typename Elem<T>::key_t;
     constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
+    constexpr int shift1 = Elem<T>::key_bits - 2 * kRadixBits;
     constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit, s_base, s_wave[kFirstBlock / 64];
@@ -332,14 +333,28 @@ __global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __re
         keys[i] = mine;
     }
     hist_add(lds_hist, have, (unsigned)(mine >> shift0) & kDigitMask);
-    if (!short_on) {
-        merge_hist<kFirstBlock>(lds_hist, st);
-    } else {
+    // (the global histogram is only read when the short list cannot decide; adding to it costs
+    // this launch under a microsecond, counting every key again in the second launch would cost 7)
+    merge_hist<kFirstBlock>(lds_hist, st);
+    if (short_on) {
         __syncthreads();
         unsigned digit;
         unsigned long long above;
         block_pick<kFirstBlock>(lds_hist, (unsigned long long)(short_k - 1), s_sum, &s_digit, &s_above, digit, above);
-        const bool out = have && ((unsigned)(mine >> shift0) & kDigitMask) >= digit;
+        // the cut is refined by the second digit: a top digit alone can be as coarse as a whole
+        // binade (64-bit keys: it is the exponent), and a block would pass on every key of it
+        for (int b = t; b < kRadixBins; b += kFirstBlock) lds_hist[b] = 0u;
+        __syncthreads();
+        const unsigned first_digit = (unsigned)(mine >> shift0) & kDigitMask;
+        const unsigned second_digit = (unsigned)(mine >> shift1) & kDigitMask;
+        hist_add(lds_hist, have && first_digit == digit, second_digit);
+        __syncthreads();
+        unsigned digit2;
+        unsigned long long above2;
+        block_pick<kFirstBlock>(lds_hist, (unsigned long long)(short_k - 1) - above, s_sum, &s_digit, &s_above, digit2,
+                                above2);
+        const unsigned cut = (digit << kRadixBits) | digit2;  // leading 2 * kRadixBits bits of the block's short_k-th key
+        const bool out = have && ((first_digit << kRadixBits) | second_digit) >= cut;
         const unsigned long long outs = __ballot(out);
         const int lane = t & 63, wave = t >> 6;
         if (lane == 0) s_wave[wave] = (unsigned)__popcll(outs);
@@ -348,7 +363,7 @@ __global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __re
             unsigned total = 0;
             for (int w = 0; w < kFirstBlock / 64; ++w) total += s_wave[w];
             s_base = atomicAdd(&st->short_count, total);
-            atomicMax(&st->short_digit, digit);
+            atomicMax(&st->short_digit, cut);
         }
         __syncthreads();
         unsigned at = s_base + (unsigned)__popcll(outs & ((1ull << lane) - 1ull));
@@ -367,13 +382,14 @@ template <typename KEY> __device__ __forceinline__ void wave_and_or(KEY& a, KEY&
     }
 }
 
-// The second launch.  A short list that fits LDS is moved there in one round trip to memory,
-// keeping only the keys from the digit on from which the list is complete.  Those keys share
-// their leading bits (they are the largest few percent): the digits are taken from the first bit
-// in which they differ, so that ONE histogram spreads them over the bins, and as soon as at most
-// kDirect keys are left the wanted one is found by counting, for each, the keys above it.
-// Everything else (no short list, a list too long for LDS, a rank the list does not reach) walks
-// the fixed digits from the top, as the whole-vector passes do.
+// The second launch.  The short list's keys from the digit on from which the list is complete move
+// to LDS (a round trip to memory per kListKeys listed keys).  Those keys share their leading bits
+// (they are the largest few percent): the digits are taken from the first bit in which they differ,
+// so that ONE histogram spreads them over the bins, and as soon as at most kDirect keys are left the
+// wanted one is found by counting, for each, the keys above it.  Everything else (no short list,
+// more such keys than LDS holds, a rank the list does not reach) starts from the first launch's
+// top-digit counts of all keys and walks the fixed digits from the top over the key array, as the
+// whole-vector passes do.
 constexpr int kDirect = 256;
 
 template <typename T>
@@ -386,8 +402,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kListKeys = kListBytes / (int)sizeof(key_t);
-    constexpr int shift0 = kKeyBits - kRadixBits;
-    constexpr unsigned kDigitMask = (1u << kRadixBits) - 1u;
+    constexpr int shift1 = kKeyBits - 2 * kRadixBits;
     constexpr key_t kAllBits = (key_t)(~(key_t)0) >> (8 * (int)sizeof(key_t) - kKeyBits);
     static_assert(kDirect * sizeof(key_t) <= kRadixBins * sizeof(unsigned), "the candidates reuse the histogram");
     __shared__ __align__(8) unsigned lds_hist[kRadixBins];
@@ -400,7 +415,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
 
     // what the first launch's blocks passed on
     const unsigned short_count = short_on ? st->short_count : 0u;
-    const unsigned short_digit = short_on ? st->short_digit : 0u;
+    const unsigned short_cut = short_on ? st->short_digit : 0u;  // leading 2 * kRadixBits bits
     for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
     if (t == 0) {
         s_fill = 0u;
@@ -419,28 +434,33 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     unsigned src_n = (unsigned)m;
     bool listed = false, counted = false;
     unsigned list_n = 0;
-    if (short_on && short_count <= (unsigned)kListKeys && short_count <= short_cap) {
+    if (short_on && short_count <= short_cap) {
+        // the listed keys from the digit on from which the list is complete move to LDS, a round
+        // trip to memory per kListKeys of them (one, usually); their order does not matter
         constexpr int kPer = kListKeys / kFinishBlock;
-        key_t kk[kPer];
-#pragma unroll
-        for (int q = 0; q < kPer; ++q) {
-            const unsigned j = (unsigned)(q * kFinishBlock + t);
-            kk[q] = j < short_count ? short_keys[j] : (key_t)0;
-        }
         key_t all_and = kAllBits, all_or = (key_t)0;
+        for (unsigned first = 0; first < short_count; first += (unsigned)(kPer * kFinishBlock)) {
+            key_t kk[kPer];
 #pragma unroll
-        for (int q = 0; q < kPer; ++q) {
-            if ((unsigned)(q * kFinishBlock) < short_count) {  // the same for the whole block
-                const unsigned j = (unsigned)(q * kFinishBlock + t);
-                const bool in = j < short_count && ((unsigned)(kk[q] >> shift0) & kDigitMask) >= short_digit;
-                const unsigned long long ins = __ballot(in);
-                unsigned base = 0;
-                if (lane == 0 && ins) base = atomicAdd(&s_fill, (unsigned)__popcll(ins));
-                base = __shfl(base, 0, 64);
-                if (in) {
-                    s_list[base + (unsigned)__popcll(ins & ((1ull << lane) - 1ull))] = kk[q];
-                    all_and &= kk[q];
-                    all_or |= kk[q];
+            for (int q = 0; q < kPer; ++q) {
+                const unsigned j = first + (unsigned)(q * kFinishBlock + t);
+                kk[q] = j < short_count ? short_keys[j] : (key_t)0;
+            }
+#pragma unroll
+            for (int q = 0; q < kPer; ++q) {
+                if (first + (unsigned)(q * kFinishBlock) < short_count) {  // the same for the whole block
+                    const unsigned j = first + (unsigned)(q * kFinishBlock + t);
+                    const bool in = j < short_count && (unsigned)(kk[q] >> shift1) >= short_cut;
+                    const unsigned long long ins = __ballot(in);
+                    unsigned base = 0;
+                    if (lane == 0 && ins) base = atomicAdd(&s_fill, (unsigned)__popcll(ins));
+                    base = __shfl(base, 0, 64);
+                    const unsigned at = base + (unsigned)__popcll(ins & ((1ull << lane) - 1ull));
+                    if (in && at < (unsigned)kListKeys) {  // (more than fit: seen from the count)
+                        s_list[at] = kk[q];
+                        all_and &= kk[q];
+                        all_or |= kk[q];
+                    }
                 }
             }
         }
@@ -451,7 +471,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         }
         __syncthreads();
         const unsigned complete = s_fill;
-        if (rank < (unsigned long long)complete) {  // the wanted key is one of these
+        if (complete <= (unsigned)kListKeys && rank < (unsigned long long)complete) {  // the wanted key is one of these
             counted = true;
             listed = true;
             list_n = complete;
@@ -461,38 +481,15 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
             mask = kAllBits & ~open_bits;
             prefix = s_and & mask;
         }
-    } else if (short_on && short_count <= short_cap) {
-        // top digits of the short list, from the digit on from which the list is complete
-        unsigned seen = 0;
-        scan_matching<key_t>(short_keys, short_count, (key_t)0, (key_t)0, [&](key_t k1) {
-            const unsigned d = (unsigned)(k1 >> shift0) & kDigitMask;
-            if (d >= short_digit) {
-                atomicAdd(&lds_hist[d], 1u);
-                ++seen;
-            }
-        });
-        if (seen) atomicAdd(&s_fill, seen);
-        __syncthreads();
-        if (rank < (unsigned long long)s_fill) {
-            counted = true;
-            src = short_keys;
-            src_n = short_count;
-        }
     }
     __syncthreads();
-    bool hist_ready = counted && !listed;
+    bool hist_ready = false;
+    // top digit of every key, counted by the first launch: used when the short list did not decide
+    for (int b = t; b < kRadixBins; b += kFinishBlock) {
+        if (!counted) lds_hist[b] = st->hist[b];
+        st->hist[b] = 0u;  // leave it clean for the next run
+    }
     if (!counted) {
-        if (short_on) {  // nobody merged counts: count the top digit of every key
-            for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
-            __syncthreads();
-            scan_matching<key_t>(keys, (unsigned)m, (key_t)0, (key_t)0,
-                                 [&](key_t k1) { atomicAdd(&lds_hist[(unsigned)(k1 >> shift0) & kDigitMask], 1u); });
-        } else {
-            for (int b = t; b < kRadixBins; b += kFinishBlock) {
-                lds_hist[b] = st->hist[b];
-                st->hist[b] = 0u;  // leave it clean for the next run
-            }
-        }
         hist_ready = true;
         __syncthreads();
     }
