@@ -49,6 +49,8 @@ constexpr unsigned kDeferred = 0x80000000u;
 #endif
 constexpr int kGatherBlock = CX_GATHER_BLOCK;  // threads of a gather block
 constexpr int kGatherTiles = 64;                // tiles a gather block owns: one lane per tile in its scan
+static_assert(kGatherTiles % (kWavesPerBlock * 8) == 0, "a gather block's streaming blocks fill whole 16-byte loads of 16-bit sums");
+static_assert(kWavesPerBlock * 64 * 4 * 16 <= 65535, "a streaming block's survivors fit 16 bits (largest tile: 64 lanes x 16 loads x 4 elements)");
 
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
@@ -276,7 +278,10 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
                                         : (unsigned)kWavesPerBlock;
         atomicAdd(&s_sum, total);  // LDS
         __threadfence_block();
-        if (atomicAdd(&s_done, 1u) == tiles_here - 1u) block_sums[block] = atomicAdd(&s_sum, 0u);
+        // 16 bits per sum (a block has at most a few thousand elements): every gather block reads
+        // all the sums before its own, and halving them shortens that read
+        if (atomicAdd(&s_done, 1u) == tiles_here - 1u)
+            reinterpret_cast<unsigned short*>(block_sums)[block] = (unsigned short)atomicAdd(&s_sum, 0u);
     }
 }
 
@@ -323,12 +328,14 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     unsigned before = 0;
     {
         // stage blocks before this block's first tile: kGatherTiles / kWavesPerBlock per gather block
+        // (eight 16-bit sums per 16-byte load)
         const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
-        const unsigned nvec = blockIdx.x * (kGatherTiles / kWavesPerBlock / 4);
+        const unsigned nvec = blockIdx.x * (kGatherTiles / kWavesPerBlock / 8);
 #pragma unroll 8
         for (unsigned v = tid; v < nvec; v += kGatherBlock) {
             const uint4 c = b4[v];
-            before += c.x + c.y + c.z + c.w;
+            before += (c.x & 0xffffu) + (c.x >> 16) + (c.y & 0xffffu) + (c.y >> 16) + (c.z & 0xffffu) + (c.z >> 16) +
+                      (c.w & 0xffffu) + (c.w >> 16);
         }
     }
 #pragma unroll
