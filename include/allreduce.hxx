@@ -81,9 +81,7 @@ public:
         const int myRank = this->gaspi_env->get_rank();
         const int numRanks = this->gaspi_env->get_ranks();
         if (myRank == chiefRank) {
-            // reduce in ascending rank order: this fixes the order of the floating-point additions
-            for (int rank = 0; rank < numRanks; ++rank)
-                if (rank != chiefRank) comm_reduce_map[rank].readRemote_add(data, size);
+            reduce_workers(data, size);
             // broadcast: compress once, hand the same buffer to the other workers
             int copy_rank = -1;
             for (int rank = 0; rank < numRanks; ++rank) {
@@ -104,14 +102,30 @@ public:
     // workers send their residuals, the chief adds them; nothing is broadcast; everything is reset
     virtual void flush(data_t* data, int size) {
         const int myRank = this->gaspi_env->get_rank();
-        const int numRanks = this->gaspi_env->get_ranks();
         if (myRank == chiefRank) {
-            for (int rank = 0; rank < numRanks; ++rank)
-                if (rank != chiefRank) comm_reduce_map[rank].readRemote_add(data, size);
+            reduce_workers(data, size);
         } else {
             comm_reduce_map[chiefRank].flushRests();
         }
         reset();
+    }
+
+    // The chief's loop `for rank: readRemote_add(data)` (src/allreduce.tpp:186-189) as one pass over
+    // `data`: every worker's message is waited for, then all are added in ascending rank order (which
+    // fixes the order of the floating-point additions, as the loop does) by one rank-ordered reduce.
+    void reduce_workers(data_t* data, int size) {
+        const int numRanks = this->gaspi_env->get_ranks();
+        std::vector<const void*> messages;
+        int first = -1;
+        for (int rank = 0; rank < numRanks; ++rank) {
+            if (rank == chiefRank) continue;
+            messages.push_back(comm_reduce_map[rank].waiting_message());
+            if (first < 0) first = rank;
+        }
+        if (first < 0) return;
+        comm_reduce_map[first].add_messages(data, size, messages.data(), (int)messages.size());
+        for (int rank = 0; rank < numRanks; ++rank)
+            if (rank != chiefRank) comm_reduce_map[rank].message_done();
     }
 
     void reset() {

@@ -302,6 +302,19 @@ public:
         targBuff_data->consumed();
     }
 
+    // Not in the reference: a receiver that takes the messages of several channels in one call (the
+    // chief of the all-to-one schedule) waits for each, collects their device addresses, adds them all
+    // with add_messages() of one of the objects, and releases the channels with message_done().
+    const void* waiting_message() {
+        if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
+        wait_for_message();
+        return targ_address() + (send_sizeBytes ? (int)sizeof(int) : 0);
+    }
+    void message_done() { targBuff_data->consumed(); }
+    void add_messages(VarTYPE* vector, int size, const void* const* messages, int count) {
+        compressor->add_many(vector, size, messages, count);
+    }
+
     // receive, pass the compressed message on to this object's target, and decompress it
     void readRemote_forward(VarTYPE* vector, int size) {
         wait_for_message();

@@ -54,6 +54,13 @@ public:
 
     virtual Compressor<VarTYPE>* clone() const = 0;
 
+    // Not in the reference: adds `count` messages (device addresses) to `output` in the order given,
+    // which is what the chief's loop over its workers does, one add() per worker
+    // (src/allreduce.tpp:186-189); a compressor may do it in one pass over `output`.
+    virtual void add_many(VarTYPE* output, int output_size, const void* const* d_sources, int count) {
+        for (int i = 0; i < count; ++i) add(output, output_size, d_sources[i]);
+    }
+
     // Not in the reference: bytes of the largest message a vector of n elements can produce.
     virtual long long max_message_bytes(int n) const = 0;
 
@@ -211,6 +218,23 @@ protected:
         cxx::check(cx_ip_add(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_in, 0));
         o.flush();
         cxx::check(cx_synchronize(h));
+    }
+
+public:
+    // one rank-ordered pass over `output` for all the messages: each element is read and written
+    // once, the additions to it happen in the order of the messages, exactly as with one add() per
+    // message.  The kernels check every header first: a message made for a longer vector leaves
+    // `output` untouched.
+    virtual void add_many(VarTYPE* output, int output_size, const void* const* d_sources, int count) {
+        if (count <= 0) return;
+        cx_handle h = this->handle_.get();
+        cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
+        cxx::check(cx_ip_reduce(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_sources, count, 1, 0));
+        const int rc = cx_synchronize(h);
+        if (rc == CX_ERR_MSG_TOO_LARGE)
+            throw std::runtime_error("Decompression vector size is bigger than output buffer!");
+        cxx::check(rc);
+        o.flush();
     }
 };
 
