@@ -317,6 +317,16 @@ def main():
             log("reduce %s %.3f ms (%.0f GB/s of 4n+16Rk, %.1f%% of peak)"
                 % (name, r_ms, reduce[name + "_GBps"], 100 * reduce[name + "_frac"]))
         reduce["pairs_per_s"] = len(msgs) * c5k / (reduce["ordered_ms"] * 1e-3)
+        # the chief's own form of the loop: the messages are added INTO its vector (readRemote_add per
+        # worker), so every element is read and written: 8n + 16Rk bytes
+        acc_bytes = 8 * c5n + 16 * len(msgs) * c5k
+        for _ in range(2):
+            h.reduce(dense, msgs, accumulate=True, mode=0)
+        acc_ms = event_ms(torch, lambda: h.reduce(dense, msgs, accumulate=True, mode=0), reps)
+        reduce["accumulate"] = {"algorithmic_bytes": acc_bytes, "ms": acc_ms, "GBps": acc_bytes / (acc_ms * 1e-3) / 1e9,
+                                "frac": acc_bytes / (acc_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        log("reduce ordered, added into the vector %.3f ms (%.0f GB/s of 8n+16Rk, %.1f%% of peak)"
+            % (acc_ms, reduce["accumulate"]["GBps"], 100 * reduce["accumulate"]["frac"]))
         # residual apply (K4): rests += dense, 12 bytes per element
         c5_rests = torch.zeros(c5n, device="cuda")
         for _ in range(2):

@@ -340,6 +340,16 @@ constexpr int kMergeWaves = CX_MERGE_WAVES;        // message wavefronts of a bl
 constexpr int kWriterWaves = CX_WRITER_WAVES;      // wavefronts that stream finished tiles out
 constexpr int kMergeBlock = 64 * (kMergeWaves + kWriterWaves);
 constexpr int kMergeBufs = kMergeWaves + 1;        // LDS tiles of a block: one per pipeline stage
+// Adding into an existing vector: LOADER wavefronts bring a tile's old contents into its LDS buffer
+// two steps before the first message wavefront gets there (asynchronous global-to-LDS loads in a
+// queue of their own: a wavefront that also stores would wait for its stores with every load),
+// which takes two more buffers.
+constexpr int kLoaderWaves = 4;
+constexpr int kPrefillAhead = 2;
+template <bool ACCUM> struct MergeShape {
+    static constexpr int bufs = ACCUM ? kMergeBufs + kPrefillAhead : kMergeBufs;
+    static constexpr int block = kMergeBlock + (ACCUM ? 64 * kLoaderWaves : 0);
+};
 constexpr int kMsgsPerWave = kMergeMsgs / kMergeWaves;
 template <typename T> struct MergeTile { static constexpr int value = CX_MERGE_TILE_BYTES / (int)sizeof(T); };
 #ifndef CX_MERGE_NT
@@ -468,7 +478,7 @@ __device__ __forceinline__ unsigned lane_below(unsigned v, unsigned first) {
 // next); they never load (unless accumulating), so the stores of many tiles are in flight per
 // block.  kMergeBufs LDS tiles rotate; one barrier per step.
 template <typename T, int OP, bool ACCUM>
-__global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out, int out_n, MergeList list,
+__global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __restrict__ out, int out_n, MergeList list,
                                                             int n_msgs, unsigned ntiles, unsigned tiles_per_block,
                                                             DeviceStatus* status) {
     constexpr int PW = Elem<T>::pair_words;
@@ -479,11 +489,13 @@ __global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out,
     constexpr int kWriters = kMergeBlock - 64 * kMergeWaves;      // writer threads
     constexpr int kVecs = kTile / VEC / kWriters;                  // 16-byte vectors a writer thread moves per tile
     static_assert(kVecs * kWriters * VEC == kTile, "the writers cover a tile exactly");
-    __shared__ T tiles[kMergeBufs][kTile];
+    constexpr int kBufs = MergeShape<ACCUM>::bufs;
+    __shared__ T tiles[kBufs][kTile];
     __shared__ unsigned stage[kMergeWaves][kMsgsPerWave][kRingPairs * PW];  // the rings of chunks, per message
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // the same for the whole wavefront: scalar branches
-    const bool writer = wave >= kMergeWaves;
+    const bool writer = wave >= kMergeWaves && wave < kMergeWaves + kWriterWaves;
+    const bool loader = ACCUM && wave >= kMergeWaves + kWriterWaves;
     const unsigned t0 = blockIdx.x * tiles_per_block;
     if (t0 >= ntiles) return;
     const unsigned t1 = t0 + tiles_per_block < ntiles ? t0 + tiles_per_block : ntiles;
@@ -508,27 +520,59 @@ __global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out,
         return (int)(left < kTile ? left : kTile);
     };
 
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+    if (loader) {
+        // ---- loader wavefronts (accumulating only) ----
+        constexpr int kTileDwords = kTile * (int)sizeof(T) / 4;
+        constexpr int kLoadsPerWave = kTileDwords / 64 / kLoaderWaves;  // one dword per lane each
+        static_assert(kLoadsPerWave * 64 * kLoaderWaves == kTileDwords, "the loaders cover a tile exactly");
+        const int lw = wave - (kMergeWaves + kWriterWaves);
+        const unsigned* const safe = reinterpret_cast<const unsigned*>(out);  // out_n > 0: the first element exists
+        auto prefill = [&](unsigned a) {  // tile a of this block: old contents into its buffer
+            const unsigned t = t0 + a;
+            const unsigned valid_dwords = (unsigned)tile_valid(t) * (unsigned)(sizeof(T) / 4);
+            const unsigned* src = reinterpret_cast<const unsigned*>(out + (long long)t * kTile);
+            const unsigned lds = (unsigned)(uintptr_t)(lds_ptr_t)&tiles[a % (unsigned)kBufs][0];
+#pragma unroll
+            for (int c = 0; c < kLoadsPerWave; ++c) {
+                const unsigned j = (unsigned)((lw * kLoadsPerWave + c) * 64 + lane);
+                // (what lies behind the vector's end is never written out; those lanes read the first element)
+                async_load_to_lds(j < valid_dwords ? src + j : safe,
+                                  (unsigned)__builtin_amdgcn_readfirstlane((int)(lds + (unsigned)((lw * kLoadsPerWave + c) * 256))));
+            }
+        };
+        for (unsigned a = 0; a < (unsigned)kPrefillAhead && a < my_tiles; ++a) prefill(a);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+        for (unsigned s = 0; s < steps; ++s) {
+            // the buffer of tile s + kPrefillAhead was drained a step ago; the tile the first message
+            // wavefront takes next step (asked for a step ago) has landed when only this step's
+            // loads are still in flight
+            const unsigned a = s + (unsigned)kPrefillAhead;
+            if (a < my_tiles) {
+                prefill(a);
+                __builtin_amdgcn_s_waitcnt(0x0f70 | ((kLoadsPerWave & 0xf)) | ((kLoadsPerWave >> 4) << 14));
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            lds_barrier();
+        }
+        return;
+    }
     if (writer) {
         const int wt = tid - 64 * kMergeWaves;
-        // every buffer starts as zeros, or as the old contents of the tile that uses it first
-        for (int b = 0; b < kMergeBufs; ++b) {
-            const unsigned t = t0 + (unsigned)b;
-            const int valid = ACCUM ? tile_valid(t) : 0;
-            for (int i = wt; i < kTile; i += kWriters) tiles[b][i] = i < valid ? out[(long long)t * kTile + i] : (T)0;
+        if (!ACCUM) {  // every buffer starts as zeros
+            for (int b = 0; b < kBufs; ++b)
+                for (int i = wt; i < kTile; i += kWriters) tiles[b][i] = (T)0;
         }
         lds_barrier();
-        Pack<T, VEC> nxt[kVecs];  // ACCUM: old contents of the tile that takes over the buffer drained next step
         for (unsigned s = 0; s < steps; ++s) {
             const bool draining = s >= (unsigned)kMergeWaves;
             const unsigned d = s - (unsigned)kMergeWaves;  // tile (of this block) that is streamed out
-            T* dbuf = tiles[d % (unsigned)kMergeBufs];
+            T* dbuf = tiles[d % (unsigned)kBufs];
             const long long base = (long long)(t0 + d) * kTile;
             const int valid = draining ? tile_valid(t0 + d) : 0;
             const bool fast = draining && aligned && valid == kTile;
-            const unsigned heir = t0 + d + (unsigned)kMergeBufs;  // the tile that uses the buffer next
-            const bool refill = ACCUM && draining && heir < t1;
-            const bool refill_fast = refill && aligned && tile_valid(heir) == kTile;
-            const bool ahead = ACCUM && s + 1u >= (unsigned)kMergeWaves && aligned && tile_valid(heir + 1u) == kTile;
 #pragma unroll
             for (int q = 0; q < kVecs; ++q) {
                 const int e = (q * kWriters + wt) * VEC;
@@ -544,23 +588,12 @@ __global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out,
                     for (int c = 0; c < VEC; ++c)
                         if (e + c < valid) out[base + e + c] = dbuf[e + c];
                 }
-                if (draining) {
-                    // what the buffer's next tile starts from
+                if (draining && !ACCUM) {  // the buffer's next tile starts from zeros (the loaders fill it otherwise)
                     Pack<T, VEC> z;
 #pragma unroll
                     for (int c = 0; c < VEC; ++c) z.x[c] = (T)0;
-                    if (refill_fast) {
-                        z = nxt[q];  // asked for a step ago
-                    } else if (refill) {
-                        const int nv = tile_valid(heir);
-#pragma unroll
-                        for (int c = 0; c < VEC; ++c)
-                            if (e + c < nv) z.x[c] = out[(long long)heir * kTile + e + c];
-                    }
                     *reinterpret_cast<Pack<T, VEC>*>(&dbuf[e]) = z;
                 }
-                if (ahead)  // for the refill one step from now
-                    nxt[q] = *reinterpret_cast<const Pack<T, VEC>*>(out + (long long)(heir + 1u) * kTile + e);
             }
             lds_barrier();
         }
@@ -659,7 +692,7 @@ __global__ __launch_bounds__(kMergeBlock) void merge_kernel(T* __restrict__ out,
         if (step >= (unsigned)wave && a < my_tiles) {
             const unsigned t = t0 + a;
             T* tile = tiles[buf];
-            buf = buf + 1u == (unsigned)kMergeBufs ? 0u : buf + 1u;
+            buf = buf + 1u == (unsigned)kBufs ? 0u : buf + 1u;
             const unsigned base = t * (unsigned)kTile;
             const unsigned valid = (unsigned)tile_valid(t);
             const unsigned tile_end = base + valid;
@@ -743,6 +776,9 @@ int check_headers(cx_handle h, const void* const* msgs, int n_msgs) {
 }
 
 template <typename T>
+int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate);
+
+template <typename T>
 int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
     if (out_n == 0) return check_headers(h, msgs, n_msgs);
     constexpr int kTile = MergeTile<T>::value;
@@ -760,11 +796,19 @@ int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n
             list.msg[r] = r < cnt ? static_cast<const unsigned*>(msgs[first + r]) : nullptr;
         const bool acc = accumulate || first > 0;
 #define CX_MERGED(OP, ACC)                                                                                        \
-    hipLaunchKernelGGL((merge_kernel<T, OP, ACC>), dim3(grid), dim3(kMergeBlock), 0, h->stream, out, out_n, list, \
+    hipLaunchKernelGGL((merge_kernel<T, OP, ACC>), dim3(grid), dim3(MergeShape<ACC>::block), 0, h->stream, out, out_n, list, \
                        cnt > 0 ? cnt : 0, ntiles, tiles_per_block, h->d_status)
-        if (op == 0) CX_MERGED(0, false);
-        else if (acc) CX_MERGED(1, true);
-        else CX_MERGED(1, false);
+        if (op == 0) {
+            CX_MERGED(0, false);
+        } else if (!acc) {
+            CX_MERGED(1, false);
+        } else if constexpr (sizeof(T) == 4) {
+            CX_MERGED(1, true);
+        } else {
+            // 8-byte elements: the rings of 12-byte pairs and seven tiles do not fit one block's LDS
+            int rc = launch_tiled<T>(h, out, out_n, msgs + first, cnt, 1, 1);
+            if (rc != CX_OK) return rc;
+        }
 #undef CX_MERGED
         if (n_msgs == 0) break;
     }
@@ -1012,14 +1056,20 @@ int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n
     if ((!out && out_n > 0) || out_n < 0 || n_msgs < 0 || (n_msgs > 0 && !msgs)) return fail(CX_ERR_INVALID, "reduce: bad arguments");
     if (out_n == 0) return check_headers(h, msgs, n_msgs);
     if (mode == 0 && h->reduce_variant == 3) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
-    if (mode == 0 && h->reduce_variant == 0 && !accumulate && n_msgs > 1) {
-        // measured on 64 Mi fp32 elements with 1 %-dense messages: writing the vector from zeros, the
-        // pipelined kernel wins from two messages on (8 messages: 62 against 87 us); adding into it,
-        // the one-block-per-tile kernel is as fast or faster (4 messages: 110 against 136 us)
-        const int head = n_msgs < kMergeMsgs ? n_msgs : kMergeMsgs;
-        int rc = launch_merged<T>(h, out, out_n, msgs, head, 1, 0);
-        if (rc != CX_OK || head == n_msgs) return rc;
-        return launch_tiled<T>(h, out, out_n, msgs + head, n_msgs - head, 1, 1);
+    if (mode == 0 && h->reduce_variant == 0) {
+        // Measured on 64 Mi fp32 elements with 1 %-dense messages, 1 / 2 / 4 / 8 messages.  Writing the
+        // vector from zeros: pipelined 53 / 48 / 54 / 63 us against one block per tile 43 / 48 / 62 / 87 us.
+        // Adding into it: pipelined (loader wavefronts) 92 / 92 / 93 / 93 us against 83 / 90 / 110 / 141 us.
+        // With 8-byte elements the accumulating pipeline does not fit a block's LDS.
+        const bool four_bytes = sizeof(T) == 4;
+        if (!accumulate && n_msgs > 1) {
+            if (four_bytes) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, 0);  // later batches of 8 add
+            const int head = n_msgs < kMergeMsgs ? n_msgs : kMergeMsgs;
+            int rc = launch_merged<T>(h, out, out_n, msgs, head, 1, 0);
+            if (rc != CX_OK || head == n_msgs) return rc;
+            return launch_tiled<T>(h, out, out_n, msgs + head, n_msgs - head, 1, 1);
+        }
+        if (accumulate && n_msgs > 2 && four_bytes) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, 1);
     }
     if (mode == 0 && (h->reduce_variant == 0 || h->reduce_variant == 2))
         return launch_tiled<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
