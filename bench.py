@@ -218,7 +218,9 @@ def main():
     for key, what, fn in (("cold", "1 GiB read by another kernel between steps (memory-side cache evicted, clean)",
                            lambda: evict.sum()),
                           ("cold_after_writes", "1 GiB rewritten by another kernel between steps (cache evicted, dirty)",
-                           lambda: evict.add_(1.0))):
+                           lambda: evict.add_(1.0)),
+                          ("gradient_rewritten", "the gradient itself rewritten in place by another kernel between steps "
+                           "(what a backward pass leaves: its tail in the cache, dirty)", lambda: g.mul_(1.0))):
         # two passes: the step is timed without the library's events around its streaming kernel
         # (each event costs the step some 3 us between two kernels), the kernel in a pass of its own
         cold_step_ms = event_ms(torch, step, cold_reps, between=fn)
