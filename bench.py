@@ -134,6 +134,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--items", type=int, default=None, help="compaction tile option (2/4/8)")
     ap.add_argument("--alternate", type=int, default=None, help="stage_alternate option (0/1)")
+    ap.add_argument("--cached-tail-mb", type=int, default=None, help="stage_cached_tail_mb option (-1 = all cacheable)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of the gradient (4n bytes read, 4n written) so that "
                          "a counter run has a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
@@ -162,6 +163,8 @@ def main():
         h.set_option("compact_items", args.items)
     if args.alternate is not None:
         h.set_option("stage_alternate", args.alternate)
+    if args.cached_tail_mb is not None:
+        h.set_option("stage_cached_tail_mb", args.cached_tail_mb)
     g = torch.from_numpy(g_h).cuda()
     idx = torch.from_numpy(idx_h).cuda()
     rests = torch.zeros(n, device="cuda")

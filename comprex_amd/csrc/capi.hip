@@ -303,6 +303,8 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->profile_tick = 0;
     } else if (!strcmp(key, "stage_alternate")) {
         h->stage_alternate = value ? 1 : 0;
+    } else if (!strcmp(key, "stage_cached_tail_mb")) {
+        h->stage_cached_tail_mb = value < 0 ? -1 : value;
     } else if (!strcmp(key, "select_bracket")) {
         h->select_bracket = value ? 1 : 0;
     } else if (!strcmp(key, "reduce_variant")) {
@@ -325,6 +327,7 @@ int cx_get_option(cx_handle h, const char* key, int* value) {
     if (!strcmp(key, "compact_items")) *value = h->compact_items;
     else if (!strcmp(key, "profile_stage")) *value = h->profile;
     else if (!strcmp(key, "stage_alternate")) *value = h->stage_alternate;
+    else if (!strcmp(key, "stage_cached_tail_mb")) *value = h->stage_cached_tail_mb;
     else if (!strcmp(key, "select_bracket")) *value = h->select_bracket;
     else if (!strcmp(key, "reduce_variant")) *value = h->reduce_variant;
     else if (!strcmp(key, "reduce_blocks_per_cu")) *value = h->reduce_blocks_per_cu;

@@ -123,6 +123,7 @@ struct cx_handle_s {
     // options
     int compact_items = 4;             // 16-byte loads per lane and tile
     int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
+    int stage_cached_tail_mb = 192;    // residual read cacheably over the last so many MB of a walk (-1: all of it)
     int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound
     int select_short_list = 1;         // 1 = the two-launch select passes a short list of top keys to its second launch
     int fused_topk = 1;                // 1 = cx_ip_compress_topk may take its single-pass route

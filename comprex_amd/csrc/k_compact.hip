@@ -55,9 +55,14 @@ static_assert(kWavesPerBlock * 64 * 4 * 16 <= 65535, "a streaming block's surviv
 template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 
 // Cache policy of the streaming pass.  The gradient is read once per step and the residual
-// is rewritten once per step, so both bypass the caches (nontemporal); the residual's READS
-// stay cacheable, which leaves the tail of the pass in the 256 MB memory-side cache, and the
-// next launch walks the tiles in the opposite direction (stage_alternate) to start there.
+// is rewritten once per step, so both bypass the caches (nontemporal).  The residual's READS
+// stay cacheable over the last stage_cached_tail_mb (192) MB of the walk only: that tail is what the
+// 256 MB memory-side cache still holds when the next launch walks the tiles in the opposite
+// direction (stage_alternate) and starts there; earlier reads would be pushed out before anybody
+// could use them, and by allocating they push out other lines first.  Measured on 100 M fp32
+// elements (step, everything cacheable -> 192 MB tail): consecutive steps 0.214 -> 0.206 ms; after
+// another kernel read 1 GiB 0.218 -> 0.214 ms, rewrote 1 GiB 0.265 -> 0.248 ms, rewrote the
+// gradient itself 0.250 -> 0.221 ms.  (No cacheable reads at all: 0.221 / 0.223 / 0.232 / 0.224 ms.)
 #ifndef CX_NT_DATA
 #define CX_NT_DATA 1
 #endif
@@ -129,7 +134,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
                                              unsigned* __restrict__ counts,
                                              unsigned* __restrict__ redo_flag, unsigned epoch,
                                              unsigned* __restrict__ out_pairs, long long direct_pos,
-                                             long long cap_pairs, DeviceStatus* status) {
+                                             long long cap_pairs, DeviceStatus* status, bool nt_update = false) {
     constexpr int kTile = 64 * VEC * ITEMS;
     constexpr int kCap = kTile / 8;
     constexpr int PW = Elem<T>::pair_words;
@@ -149,7 +154,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
 #pragma unroll
         for (int j = 0; j < ITEMS; ++j) {
             const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
-            if (MODE != 2) uu[j] = load_pack<T, VEC>(update + e0, false);
+            if (MODE != 2) uu[j] = load_pack<T, VEC>(update + e0, nt_update);
             if (MODE != 1) dd[j] = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
             valid_mask[j] = (1u << VEC) - 1u;
         }
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
                                                        unsigned* __restrict__ staging, unsigned* __restrict__ counts,
                                                        unsigned* __restrict__ block_sums,
                                                        unsigned* __restrict__ redo_flag, unsigned epoch,
-                                                       unsigned ntiles, int reverse) {
+                                                       unsigned ntiles, int reverse, unsigned cached_from) {
     // survivors of this block's tiles, summed in LDS; the wavefront that finishes last stores
     // the sum, which spares the gather kernel a scan over every tile count
     __shared__ unsigned s_sum, s_done;
@@ -269,9 +274,15 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
     const unsigned tile = block * kWavesPerBlock + (threadIdx.x >> 6);
     if (tile >= ntiles) return;
     const T thr = thr_ptr ? *thr_ptr : thr_val;
+    // Only the last part of the walk can still be in the memory-side cache when the next launch
+    // starts there: that part of the residual is read cacheably, everything before it bypasses the
+    // caches like the gradient (a read that allocates pushes out lines that then have to be written
+    // back, which costs most when the cache is full of another kernel's dirty lines).
+    const unsigned walk_rank = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+    const bool nt_update = __builtin_amdgcn_readfirstlane((int)(walk_rank < cached_from)) != 0;
     const unsigned total = process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63,
                                                                     staging, counts, redo_flag, epoch, nullptr, 0, 0,
-                                                                    nullptr);
+                                                                    nullptr, nt_update);
     if ((threadIdx.x & 63) == 0) {
         const unsigned tiles_here = ntiles - block * kWavesPerBlock < (unsigned)kWavesPerBlock
                                         ? ntiles - block * kWavesPerBlock
@@ -532,6 +543,11 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     h->parity ^= 1u;
 
     const unsigned stage_blocks = (ntiles + kWavesPerBlock - 1) / kWavesPerBlock;
+    // tiles at the end of the walk whose residual reads may stay in the caches
+    const unsigned long long tail_tiles =
+        h->stage_cached_tail_mb < 0 ? (unsigned long long)ntiles
+                                    : ((unsigned long long)h->stage_cached_tail_mb << 20) / ((unsigned long long)kTile * sizeof(T));
+    const unsigned cached_from = tail_tiles >= ntiles ? 0u : ntiles - (unsigned)tail_tiles;
     hipEvent_t* ev = nullptr;
     if (h->profile && h->profile_events && h->profile_count < cx_handle_s::kProfileRing &&
         (h->profile_tick++ % (unsigned)h->profile) == 0u) {  // every profile-th launch
@@ -541,7 +557,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
                        (long long)n, thr_ptr, thr_val, sc.staging, sc.counts, sc.block_sums, redo_flag, h->epoch, ntiles,
-                       reverse);
+                       reverse, cached_from);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
     // give the second pass the whole GPU instead of the gather kernel's few blocks
