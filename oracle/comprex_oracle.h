@@ -28,7 +28,13 @@
  * pin): inputs containing NaN in the threshold computation (the reference's
  * nth_element comparator is not a strict weak order for NaN); topK == 0 and
  * empty vectors in ThresholdTopK (the reference converts +inf to int / dereferences
- * end()).  The oracle returns a defined value for these and says which below.
+ * end()); the magnitude of INT_MIN (std::abs of it is undefined).  The oracle returns a
+ * defined value for these and says which below.  Also unpinned, because the transport that
+ * would show it (GaspiCxx) is not part of the reference tree: where FastComprEx's
+ * initTransferPart(sizeBytes, send_offset) lands in the receiver's buffer (taken to be its
+ * front, where the un-overridden readRemote reads), and what a second flushRests in a row
+ * re-adds from the half that was already flushed (the text of src/comprEx.tpp:404-421 is
+ * followed).
  *
  * Three element types are instantiated, as in the reference's templates:
  *   f32 (float), f64 (double), i32 (int; the type the reference's tests use).
