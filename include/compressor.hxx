@@ -210,14 +210,15 @@ protected:
     virtual void add_strategy(VarTYPE* output, int output_size, const void* sourceBuffer) {
         cx_handle h = this->handle_.get();
         const void* d_in = stage_message(sourceBuffer);
-        int hdr[2];
-        read_header(d_in, hdr);
-        if (hdr[0] > output_size)  // before anything is touched, as the reference throws
-            throw std::runtime_error("Decompression vector size is bigger than output buffer!");
         cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
+        // the kernel reads the header itself: a message made for a longer vector touches nothing and
+        // is reported by the one wait below (the reference throws before it touches the output)
         cxx::check(cx_ip_add(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_in, 0));
+        const int rc = cx_synchronize(h);
+        if (rc == CX_ERR_MSG_TOO_LARGE)
+            throw std::runtime_error("Decompression vector size is bigger than output buffer!");
+        cxx::check(rc);
         o.flush();
-        cxx::check(cx_synchronize(h));
     }
 
 public:
