@@ -249,3 +249,63 @@ def test_largest_vector_an_int32_length_allows(dev):
     # whole-vector top-k: the (pos+1)-th largest magnitude is the threshold, pos = ceil_f32(n*topK) - 1
     pos = int(np.ceil(np.float32(n) * np.float32(0.01)) - np.float32(1.0))
     assert pos - 8 <= k <= pos  # ties with the threshold stay behind
+
+
+def test_largest_vector_receive_side_and_rank_ordered_reduce(dev):
+    """n = 2^31 - 1, the largest `int size` of the reference's interface (8.6 GB per fp32 vector):
+    every index, tile number and byte offset near 2^31 has to be computed in 64 bits somewhere.
+    Checked on the GPU with torch as the independent side: pair count, ascending indices including
+    the very last element, values, residual, then decompress / add / two-message reduce of the
+    message over the same length, and the sampled threshold at positions up to the last one."""
+    n = 2**31 - 1
+    free, _ = torch.cuda.mem_get_info()
+    if free < 80 * 2**30:
+        pytest.skip("needs about 80 GB of free device memory")
+    say("largest vector: generating", n, "elements")
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    g = torch.randn(n, device="cuda", generator=gen)
+    r = torch.randn(n, device="cuda", generator=gen) * 0.25
+    g[-1], r[-1] = 50.0, 0.5          # the last element is sent
+    g[0], r[0] = -40.0, 0.25          # and the first
+    s = r + g
+    thr = np.float32(2.75)            # about 0.76 % of |N(0, 1.03)|
+    want_k = int((s.abs() > float(thr)).sum().item())
+    assert 10_000_000 < want_k < 30_000_000
+    cap = 8 + 8 * (want_k + 1000)
+    msg = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    say("largest vector: compress")
+    nbytes = dev.compress(msg, g, r, thr=thr)
+    assert nbytes == 8 + 8 * want_k
+    hdr = msg[:8].view(torch.int32)
+    assert int(hdr[0]) == n and int(hdr[1]) == want_k
+    pairs = msg[8:nbytes].view(torch.int32).view(-1, 2)
+    idx = pairs[:, 0].to(torch.int64)
+    val = pairs[:, 1].contiguous().view(torch.float32)
+    assert int(idx[0]) == 0 and int(idx[-1]) == n - 1
+    assert bool((idx[1:] > idx[:-1]).all())
+    assert torch.equal(val, s[idx])
+    keep = s.abs() <= float(thr)
+    assert torch.equal(r, torch.where(keep, s, torch.zeros((), device="cuda")))
+    del keep, g
+    say("largest vector: decompress, add, reduce")
+    dense = torch.full((n,), 3.0, device="cuda")
+    assert dev.decompress(dense, msg) == nbytes
+    assert int(torch.count_nonzero(dense).item()) == int(torch.count_nonzero(val).item())
+    assert torch.equal(dense[idx], val) and float(dense[-1]) == 50.5
+    dev.add(dense, msg)
+    assert torch.equal(dense[idx], val + val)
+    dev.reduce(dense, [msg, msg, msg], accumulate=False, mode=0)
+    dev.synchronize()
+    assert torch.equal(dense[idx], (val + val) + val)
+    assert int(torch.count_nonzero(dense).item()) == int(torch.count_nonzero(val).item())
+    dev.reduce(dense, [msg, msg, msg], accumulate=True, mode=0)
+    dev.synchronize()
+    assert torch.equal(dense[idx], ((((val + val) + val) + val) + val) + val)
+    del dense
+    say("largest vector: sampled threshold")
+    pos = torch.cat([torch.randint(0, n, (49_998,), device="cuda", generator=gen),
+                     torch.tensor([0, n - 1], device="cuda")]).to(torch.int32)
+    got = dev.topk_threshold_indexed(r, s, pos, np.float32(0.01))
+    sample = (r[pos.to(torch.int64)] + s[pos.to(torch.int64)]).abs()
+    want = float(torch.sort(sample, descending=True).values[int(np.ceil(np.float32(50_000) * np.float32(0.01))) - 1])
+    assert got == want
