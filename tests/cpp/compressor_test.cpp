@@ -109,6 +109,30 @@ template <typename data_t> int run(const char* name) {
         for (auto e : small2) if (e != 5) ++errors;  // untouched
         failed += print_pass(errors);
     }
+    {  // add_many: one pass for several messages == one add() per message, in order
+        int errors = 0;
+        CompressorIndexPairs<data_t> compressor;
+        cxx::Handle copier;
+        cxx::DeviceBuffer on_device[3];
+        const void* messages[3];
+        std::vector<data_t> one_by_one(size), at_once(size);
+        for (int i = 0; i < size; ++i) one_by_one[i] = at_once[i] = (data_t)(3 * i - 50);
+        for (int m = 0; m < 3; ++m) {
+            const int bytes = compressor.compress(buffer, values.data(), size, (data_t)(2 * m));
+            cxx::check(cx_copy(copier.get(), on_device[m].reserve((size_t)bytes), buffer, (size_t)bytes));
+            messages[m] = on_device[m].data();
+            compressor.add(one_by_one.data(), size, buffer);
+        }
+        compressor.add_many(at_once.data(), size, messages, 3);
+        for (int i = 0; i < size; ++i) if (one_by_one[i] != at_once[i]) ++errors;
+        std::vector<data_t> small(size - 1, (data_t)5);
+        try { compressor.add_many(small.data(), size - 1, messages, 3); ++errors; } catch (const std::runtime_error&) {}
+        for (auto e : small) if (e != 5) ++errors;  // untouched
+        compressor.add_many(at_once.data(), size, messages, 0);  // nothing to add
+        for (int i = 0; i < size; ++i) if (one_by_one[i] != at_once[i]) ++errors;
+        std::cout << "add_many (" << name << ")" << std::endl;
+        failed += print_pass(errors);
+    }
     {  // clones are independent objects that give the same bytes
         int errors = 0;
         CompressorIndexPairs<data_t> compressor;
