@@ -314,15 +314,16 @@ __global__ __launch_bounds__(kBlock) void tiled_kernel(T* __restrict__ out, int 
 
 // ---- merged, rank-ordered reduce: persistent blocks, no bounds pass ---------------------------
 // out (+)= sum of up to kMergeMsgs index-sorted messages, applied in the order given, the dense
-// vector written exactly once.  A block owns a CONTIGUOUS run of dense tiles; a wavefront owns two
-// of the messages.  At its start the wavefront finds, with 64-way searches, where the block's
-// index range begins and ends in its two messages; from then on it walks them with a cursor:
-// a WINDOW of 63 upcoming pairs sits in registers (lane 0 holds the pair before the cursor, for
-// the order check), the pairs below the tile's end are applied to the LDS tile, the cursor moves
-// on and the next window is fetched while the other wavefronts take their turns and the tile is
-// streamed out.  So the only memory round trips a tile waits for were started a whole tile earlier.
-// Order of additions: the wavefronts take turns (message 0,1 | 2,3 | 4,5 | 6,7) between barriers
-// that wait for LDS only, never for the stores still in flight.
+// vector written exactly once.  A block owns a CONTIGUOUS run of dense tiles; a message wavefront
+// owns two of the messages.  At its start the wavefront finds, with 16-ary searches by its quarters,
+// where the block's index range begins and ends in its two messages; from then on it walks them
+// with a cursor: the slice streams through a ring of chunks in LDS, filled by asynchronous
+// global-to-LDS loads a few chunks ahead of the cursor; each turn the wavefront looks at the 64
+// pairs from the cursor on (lane 0 also at the pair before, for the order check), applies those
+// below the tile's end to the LDS tile and moves the cursor.  So the only memory round trips a tile
+// waits for were started several tiles earlier.
+// Order of additions: the wavefronts apply messages 0,1 | 2,3 | 4,5 | 6,7 to a tile in consecutive
+// steps, between barriers that wait for LDS only, never for the stores still in flight.
 // Every pair of a message is looked at by exactly one block (the blocks' slices tile [0, k) by
 // position), so a message that is not index-sorted, or holds an index outside the vector, is
 // noticed: CX_ERR_INDEX, and no access leaves the tile.
@@ -472,11 +473,12 @@ __device__ __forceinline__ unsigned lane_below(unsigned v, unsigned first) {
 // A block is a pipeline over its tiles.  MESSAGE wavefront w (kMergeWaves of them, two messages
 // each) adds its pairs to tile s - w in step s, so the additions to one tile happen in message order,
 // one wavefront per step, while the wavefronts all work at once, on different tiles.  They never
-// store to global memory and never wait for it, except for a window that has been on its way for
+// store to global memory and never wait for it, except for a chunk that has been on its way for
 // several tiles.  WRITER wavefronts stream out the tile the last message wavefront finished a step
-// ago and leave its LDS buffer zeroed (or filled with the old contents of the tile that will use it
-// next); they never load (unless accumulating), so the stores of many tiles are in flight per
-// block.  kMergeBufs LDS tiles rotate; one barrier per step.
+// ago and, when nothing is accumulated, leave its LDS buffer zeroed; they never load, so the stores
+// of many tiles are in flight per block.  When accumulating, LOADER wavefronts fill a buffer with the
+// old contents of the tile that uses it next, kPrefillAhead steps before the first message wavefront
+// gets there.  MergeShape<ACCUM>::bufs LDS tiles rotate; one barrier per step.
 template <typename T, int OP, bool ACCUM>
 __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __restrict__ out, int out_n, MergeList list,
                                                             int n_msgs, unsigned ntiles, unsigned tiles_per_block,
