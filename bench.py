@@ -279,6 +279,19 @@ def main():
         extra["exact_topk_GBps"] = (20 * n + 8 * kx + 8) / (ex_ms * 1e-3) / 1e9
         extra["exact_topk_k"] = kx
         log("exact top-k step %.3f ms (%.0f GB/s of 20n+8k+8), k=%d" % (ex_ms, extra["exact_topk_GBps"], kx))
+        # the exact threshold alone (one read of both vectors: 8n bytes), on the residual those steps left
+        for _ in range(2):
+            h.topk_threshold(rests, g, topk, ds, to_host=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            h.topk_threshold(rests, g, topk, ds, to_host=False)
+        torch.cuda.synchronize()
+        et_ms = (time.perf_counter() - t0) / reps * 1e3
+        extra["exact_threshold_ms"] = et_ms
+        extra["exact_threshold_GBps"] = 8 * n / (et_ms * 1e-3) / 1e9
+        log("exact threshold alone %.3f ms (%.0f GB/s of 8n, %.1f%% of peak)"
+            % (et_ms, extra["exact_threshold_GBps"], 100 * extra["exact_threshold_GBps"] / HBM_PEAK_GBPS))
         # the same as one call: exact threshold and compress in a single pass over the vectors
         rests.zero_()
         for _ in range(2):
