@@ -138,10 +138,8 @@ __global__ __launch_bounds__(64) void sequential_kernel(T* out, int out_n,
 //                  collide), and is streamed out.
 // Traffic: 4 B per dense element written (+4 read when accumulating) + 8 B per pair, against
 // one read-modify-write of a scattered 4-byte element per pair for the per-message scatter.
-#ifndef CX_REDUCE_TILE_BYTES
-#define CX_REDUCE_TILE_BYTES 16384
-#endif
-template <typename T> struct ReduceTile { static constexpr int value = CX_REDUCE_TILE_BYTES / (int)sizeof(T); };
+// (tiles of 8 / 32 / 48 KB in this design measured 140 / 95 / 99 us against 93 us on 64 Mi elements)
+template <typename T> struct ReduceTile { static constexpr int value = 16384 / (int)sizeof(T); };
 constexpr int kMaxMsgs = 16;
 
 struct MsgList {
@@ -315,47 +313,51 @@ __global__ __launch_bounds__(kBlock) void tiled_kernel(T* __restrict__ out, int 
 // ---- merged, rank-ordered reduce: persistent blocks, no bounds pass ---------------------------
 // out (+)= sum of up to kMergeMsgs index-sorted messages, applied in the order given, the dense
 // vector written exactly once.  A block owns a CONTIGUOUS run of dense tiles; a message wavefront
-// owns two of the messages.  At its start the wavefront finds, with 16-ary searches by its quarters,
-// where the block's index range begins and ends in its two messages; from then on it walks them
-// with a cursor: the slice streams through a ring of chunks in LDS, filled by asynchronous
+// owns one or two of the messages.  At its start the wavefront finds (two memory round trips, all
+// its searches side by side) where the block's index range begins and ends in its messages; from
+// then on it walks them with a cursor: the slice streams through a ring of chunks in LDS, filled by asynchronous
 // global-to-LDS loads a few chunks ahead of the cursor; each turn the wavefront looks at the 64
 // pairs from the cursor on (lane 0 also at the pair before, for the order check), applies those
 // below the tile's end to the LDS tile and moves the cursor.  So the only memory round trips a tile
 // waits for were started several tiles earlier.
-// Order of additions: the wavefronts apply messages 0,1 | 2,3 | 4,5 | 6,7 to a tile in consecutive
-// steps, between barriers that wait for LDS only, never for the stores still in flight.
+// Order of additions: the wavefronts apply messages 0 | 1 | ... | 7 (or 0,1 | 2,3 | 4,5 | 6,7) to a tile
+// in consecutive steps, between barriers that wait for LDS only, never for the stores still in flight.
 // Every pair of a message is looked at by exactly one block (the blocks' slices tile [0, k) by
 // position), so a message that is not index-sorted, or holds an index outside the vector, is
 // noticed: CX_ERR_INDEX, and no access leaves the tile.
 constexpr int kMergeMsgs = 8;
-#ifndef CX_MERGE_WAVES
-#define CX_MERGE_WAVES 4
-#endif
-#ifndef CX_MERGE_TILE_BYTES
-#define CX_MERGE_TILE_BYTES 16384
-#endif
-constexpr int kMergeWaves = CX_MERGE_WAVES;        // message wavefronts of a block
-#ifndef CX_WRITER_WAVES
-#define CX_WRITER_WAVES 8
-#endif
-constexpr int kWriterWaves = CX_WRITER_WAVES;      // wavefronts that stream finished tiles out
-constexpr int kMergeBlock = 64 * (kMergeWaves + kWriterWaves);
-constexpr int kMergeBufs = kMergeWaves + 1;        // LDS tiles of a block: one per pipeline stage
 // Adding into an existing vector: LOADER wavefronts bring a tile's old contents into its LDS buffer
 // two steps before the first message wavefront gets there (asynchronous global-to-LDS loads in a
 // queue of their own: a wavefront that also stores would wait for its stores with every load),
 // which takes two more buffers.
-constexpr int kLoaderWaves = 4;
 constexpr int kPrefillAhead = 2;
-template <bool ACCUM> struct MergeShape {
-    static constexpr int bufs = ACCUM ? kMergeBufs + kPrefillAhead : kMergeBufs;
-    static constexpr int block = kMergeBlock + (ACCUM ? 64 * kLoaderWaves : 0);
+// Shape of the pipeline for element type T, writing from zeros or adding into the vector.  All of
+// a compute unit's 160 KB of LDS go to one block: tiles of 16 KB, one per pipeline stage, plus a
+// ring of chunks per message.
+//   4-byte elements from zeros: one message per message wavefront (8 stages), rings of 4 x 64 pairs:
+//     9 x 16 KB + 8 x 2 KB = 160 KB.  Measured on 64 Mi elements, 8 messages of 1 %: 51 us, against
+//     65 us with two messages per wavefront (4 stages; a wavefront's turn costs ~800 cycles whatever
+//     it finds, and the two turns of a step were the block's critical path), 77 us with 8 stages of
+//     8 KB tiles, 72 us with 8 KB tiles and two blocks per compute unit, 104 us with 4 KB tiles.
+//   adding (4 more loader wavefronts, 2 more buffers) and 8-byte elements (12-byte pairs): two
+//     messages per wavefront; rings of 4 x 128 pairs for 4-byte elements adding (144 KB) and for
+//     8-byte elements from zeros (128 KB), 4 x 64 pairs for 8-byte elements adding (136 KB; with
+//     8 KB tiles instead: 118 us against 97 us).
+//   Writer wavefronts: 4 when writing from zeros (52 us against 59 us with 8, 69 us with 2: the
+//     stores of more wavefronts queue up behind each other), 8 when adding (no difference there).
+template <typename T, bool ACCUM> struct MergeCfg {
+    static constexpr bool wide = !ACCUM && sizeof(T) == 4;  // one message per message wavefront
+    static constexpr int msg_waves = wide ? 8 : 4;
+    static constexpr int writer_waves = ACCUM ? 8 : 4;
+    static constexpr int loader_waves = ACCUM ? 4 : 0;
+    static constexpr int msgs_per_wave = kMergeMsgs / msg_waves;
+    static constexpr int tile = 16384 / (int)sizeof(T);     // elements of a tile
+    static constexpr int bufs = msg_waves + 1 + (ACCUM ? kPrefillAhead : 0);
+    static constexpr int block = 64 * (msg_waves + writer_waves + loader_waves);
+    static constexpr int chunk = (wide || (ACCUM && sizeof(T) == 8)) ? 64 : 128;  // pairs per chunk of a ring
+    static constexpr int ring_chunks = 4;
+    static constexpr int ring_pairs = chunk * ring_chunks;
 };
-constexpr int kMsgsPerWave = kMergeMsgs / kMergeWaves;
-template <typename T> struct MergeTile { static constexpr int value = CX_MERGE_TILE_BYTES / (int)sizeof(T); };
-#ifndef CX_MERGE_NT
-#define CX_MERGE_NT 1
-#endif
 
 struct MergeList {
     const unsigned* msg[kMergeMsgs];
@@ -386,64 +388,111 @@ __device__ __forceinline__ void async_load_to_lds(const unsigned* src, unsigned 
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Four lower bounds at once, by one wavefront: the 16 lanes of quarter q look for the first
-// position j in [0, k) of their message with index(j) >= target (unsigned compare), k if there is
-// none; every lane of the quarter ends up with the answer.  Each round probes 16 evenly spaced
-// positions of every bracket with independent loads, so a round costs one memory round trip for
-// all four searches and touches 16 cache lines per search.  The first bracket is a guess (indices
-// spread evenly over [0, n_hint)), checked by two extra probes in the same round.  On a message
-// that is not sorted the result is some position in [0, k]; the caller notices the disorder.
-template <int PW>
-__device__ __forceinline__ unsigned quarter_lower_bound(const unsigned* __restrict__ pairs, unsigned k, unsigned target,
-                                                        unsigned n_hint, int lane) {
-    const int sub = lane & 15, shift = lane & 48;
-    unsigned lo = 0u, hi = k;
-    bool guessed = false;
-    if (k > 16384u && n_hint > 0u && target <= n_hint) {
-        const unsigned long long g = (unsigned long long)target * k / n_hint;
-        const unsigned long long w = 2048ull;
-        lo = g > w ? (unsigned)(g - w) : 0u;
-        hi = g + w < (unsigned long long)k ? (unsigned)(g + w) : k;
-        guessed = true;
+// NS (at most four) lower bounds at once, by one wavefront: for each search s the first position j
+// in [0, k[s]) of its message with index(j) >= target[s] (unsigned compare), k[s] if there is none.
+// While a bracket is wider than 256 pairs, the 16 lanes of quarter s probe 16 evenly spaced
+// positions of it (one memory round trip for all searches, 16 cache lines per search); then every
+// bracket is read whole by the wavefront (four coalesced loads per lane: 16 cache lines) and the
+// pairs below the target are counted.  The first bracket is a guess (indices spread evenly over
+// [0, n_hint)), checked by two extra probes in the same round: two round trips then.  No load sits
+// in a branch (a load whose result is merged behind a branch is waited for at the branch, and the
+// searches would take their round trips one after the other): lanes with nothing to ask read a
+// pair of their own bracket, or `safe` when there is no message.  Positions fit 32 bits (k < 2^31).
+// The result depends on the message and the target only, so two blocks that look for the same
+// boundary agree, also on a message that is not sorted (where it is just some position in [0, k];
+// the callers notice the disorder).
+template <int PW, int NS>
+__device__ __forceinline__ void wave_lower_bound(const unsigned* const (&pairs)[NS], const unsigned (&k)[NS],
+                                                 const unsigned (&target)[NS], unsigned n_hint, int lane,
+                                                 const unsigned* safe, unsigned (&found)[NS]) {
+    static_assert(NS >= 1 && NS <= 4, "one quarter of the wavefront probes for each search");
+    constexpr unsigned kCountSpan = 256u;
+    const unsigned sub = (unsigned)lane & 15u;
+    const int quarter = lane >> 4;
+    unsigned lo[NS], hi[NS];
+    bool guessed[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        lo[s] = 0u;
+        hi[s] = k[s];
+        guessed[s] = false;
+        if (k[s] > 16384u && n_hint > 0u && target[s] <= n_hint) {
+            const unsigned g = (unsigned)((unsigned long long)target[s] * k[s] / n_hint);  // <= k
+            lo[s] = g > 2048u ? g - 2048u : 0u;
+            hi[s] = k[s] - g > 2048u ? g + 2048u : k[s];
+            guessed[s] = true;
+        }
     }
     for (int round = 0; round < 64; ++round) {  // 16-fold narrowing: a handful of rounds; bounded all the same
-        if (!__any(lo < hi || guessed)) break;
-        const unsigned span = hi - lo;
-        unsigned step = (span + 15u) / 16u;
-        if (step == 0u) step = 1u;
-        const unsigned long long pos = (unsigned long long)lo + (unsigned long long)sub * step;
-        const bool valid = pos < (unsigned long long)hi;
-        const unsigned val = valid ? pairs[(size_t)pos * PW] : 0xffffffffu;
-        // the guess holds when the pair before the bracket is below the target (lane 0 of the quarter
-        // looks) and the pair at its end is not (lane 1 looks)
-        bool chk = true;
-        if (guessed) {
-            if (sub == 0 && lo > 0u) chk = pairs[(size_t)(lo - 1u) * PW] < target;
-            if (sub == 1 && hi < k) chk = pairs[(size_t)hi * PW] >= target;
+        bool wide = false;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) wide |= guessed[s] || hi[s] - lo[s] > kCountSpan;
+        if (!__any(wide)) break;
+        unsigned step[NS], val[NS], edge[NS];
+        bool probing[NS], valid[NS], edge_lo[NS], edge_hi[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const unsigned span = hi[s] - lo[s];
+            probing[s] = guessed[s] || span > kCountSpan;
+            step[s] = (span + 15u) >> 4;
+            const unsigned* const idle = k[s] > 0u ? pairs[s] + (size_t)(lo[s] < k[s] ? lo[s] : k[s] - 1u) * PW : safe;
+            const unsigned pos = lo[s] + sub * step[s];  // < 2^32: span < 2^31
+            valid[s] = probing[s] && quarter == s && pos < hi[s];
+            val[s] = *(valid[s] ? pairs[s] + (size_t)pos * PW : idle);
+            // the guess holds when the pair before the bracket is below the target (lane 0 of the
+            // quarter looks) and the pair at its end is not (lane 1 looks)
+            edge_lo[s] = guessed[s] && quarter == s && sub == 0u && lo[s] > 0u;
+            edge_hi[s] = guessed[s] && quarter == s && sub == 1u && hi[s] < k[s];
+            edge[s] = *(edge_lo[s] ? pairs[s] + (size_t)(lo[s] - 1u) * PW
+                                   : edge_hi[s] ? pairs[s] + (size_t)hi[s] * PW : idle);
         }
-        const unsigned good = (unsigned)(__ballot(chk) >> shift) & 0xffffu;
-        const unsigned ge = (unsigned)(__ballot(!valid || val >= target) >> shift) & 0xffffu;
-        if (guessed) {
-            guessed = false;
-            if (good != 0xffffu) {  // wrong guess: search the whole message
-                lo = 0u;
-                hi = k;
-                continue;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            const bool chk = edge_lo[s] ? edge[s] < target[s] : edge_hi[s] ? edge[s] >= target[s] : true;
+            const unsigned good = (unsigned)(__ballot(chk) >> (16 * s)) & 0xffffu;
+            const unsigned ge = (unsigned)(__ballot(!valid[s] || val[s] >= target[s]) >> (16 * s)) & 0xffffu;
+            if (!probing[s]) continue;
+            if (guessed[s]) {
+                guessed[s] = false;
+                if (good != 0xffffu) {  // wrong guess: search the whole message
+                    lo[s] = 0u;
+                    hi[s] = k[s];
+                    continue;
+                }
+            }
+            const unsigned f = ge ? (unsigned)__ffs((int)ge) - 1u : 16u;  // first probe at or above the target
+            const unsigned base = lo[s];
+            if (f < 16u) {
+                const unsigned pf = base + f * step[s];
+                if (pf < hi[s]) hi[s] = pf;
+            }
+            if (f > 0u) {
+                const unsigned pl = base + (f - 1u) * step[s] + 1u;
+                lo[s] = pl < hi[s] ? pl : hi[s];
             }
         }
-        if (lo >= hi) continue;
-        const int f = ge ? __ffs((int)ge) - 1 : 16;  // first probe at or above the target
-        const unsigned base = lo;
-        if (f < 16) {
-            const unsigned long long pf = (unsigned long long)base + (unsigned long long)f * step;
-            if (pf < (unsigned long long)hi) hi = (unsigned)pf;
-        }
-        if (f > 0) {
-            const unsigned long long pl = (unsigned long long)base + (unsigned long long)(f - 1) * step + 1ull;
-            lo = pl < (unsigned long long)hi ? (unsigned)pl : hi;
+    }
+    // every bracket holds at most 256 pairs now: those below the target are counted
+    unsigned cidx[NS][4];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const unsigned* const idle = k[s] > 0u ? pairs[s] + (size_t)(lo[s] < k[s] ? lo[s] : k[s] - 1u) * PW : safe;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned p = lo[s] + (unsigned)(lane + 64 * j);
+            cidx[s][j] = *(p < hi[s] ? pairs[s] + (size_t)p * PW : idle);
         }
     }
-    return lo < hi ? lo : hi;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        unsigned cnt = 0u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned p = lo[s] + (unsigned)(lane + 64 * j);
+            cnt += (unsigned)__popcll(__ballot(p < hi[s] && cidx[s][j] < target[s]));
+        }
+        found[s] = lo[s] + cnt;
+    }
 }
 
 // A message wavefront's view of one message: a ring of chunks of kChunk pairs each in
@@ -451,15 +500,6 @@ __device__ __forceinline__ unsigned quarter_lower_bound(const unsigned* __restri
 // a saturated write stream a read takes several microseconds, far more than a tile's turn, and
 // chunks lie at fixed positions, so they can be asked for long before the cursor gets there).  Each
 // turn the wavefront looks at the 64 pairs from the cursor on, one per lane.
-constexpr int kChunk = 128;
-#ifndef CX_RING_BYTES
-#define CX_RING_BYTES 4096
-#endif
-// chunks per ring: as many as fit CX_RING_BYTES per message (a power of two, at least 4)
-template <int PW> struct Ring {
-    static constexpr int chunks = CX_RING_BYTES / (kChunk * PW * 4) >= 8 ? 8 : 4;
-    static constexpr int pairs = kChunk * chunks;
-};
 constexpr unsigned kNoPair = 0xffffffffu;  // stands for a pair behind the end of the slice
 
 // The index of the lane below (lane 0: `first`), without a trip through LDS.
@@ -470,28 +510,32 @@ __device__ __forceinline__ unsigned lane_below(unsigned v, unsigned first) {
 // OP 0: out = scatter of the (single) message, the last pair of a run of equal indices wins;
 // OP 1: out (+)= messages in order (without ACCUM: added to zeros).
 //
-// A block is a pipeline over its tiles.  MESSAGE wavefront w (kMergeWaves of them, two messages
-// each) adds its pairs to tile s - w in step s, so the additions to one tile happen in message order,
+// A block is a pipeline over its tiles.  MESSAGE wavefront w (MergeCfg::msg_waves of them, one
+// or two messages each) adds its pairs to tile s - w in step s, so the additions to one tile happen in message order,
 // one wavefront per step, while the wavefronts all work at once, on different tiles.  They never
 // store to global memory and never wait for it, except for a chunk that has been on its way for
 // several tiles.  WRITER wavefronts stream out the tile the last message wavefront finished a step
 // ago and, when nothing is accumulated, leave its LDS buffer zeroed; they never load, so the stores
 // of many tiles are in flight per block.  When accumulating, LOADER wavefronts fill a buffer with the
 // old contents of the tile that uses it next, kPrefillAhead steps before the first message wavefront
-// gets there.  MergeShape<ACCUM>::bufs LDS tiles rotate; one barrier per step.
+// gets there.  MergeCfg::bufs LDS tiles rotate; one barrier per step.
 template <typename T, int OP, bool ACCUM>
-__global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __restrict__ out, int out_n, MergeList list,
+__global__ __launch_bounds__((MergeCfg<T, ACCUM>::block)) void merge_kernel(T* __restrict__ out, int out_n, MergeList list,
                                                             int n_msgs, unsigned ntiles, unsigned tiles_per_block,
                                                             DeviceStatus* status) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int VEC = 16 / (int)sizeof(T);
-    constexpr int kTile = MergeTile<T>::value;
-    constexpr int kRingChunks = Ring<PW>::chunks;
-    constexpr int kRingPairs = Ring<PW>::pairs;
-    constexpr int kWriters = kMergeBlock - 64 * kMergeWaves;      // writer threads
+    typedef MergeCfg<T, ACCUM> Cfg;
+    constexpr int kMergeWaves = Cfg::msg_waves, kWriterWaves = Cfg::writer_waves, kLoaderWaves = Cfg::loader_waves;
+    constexpr int kMsgsPerWave = Cfg::msgs_per_wave;
+    constexpr int kChunk = Cfg::chunk;
+    constexpr int kTile = Cfg::tile;
+    constexpr int kRingChunks = Cfg::ring_chunks;
+    constexpr int kRingPairs = Cfg::ring_pairs;
+    constexpr int kWriters = 64 * kWriterWaves;      // writer threads
     constexpr int kVecs = kTile / VEC / kWriters;                  // 16-byte vectors a writer thread moves per tile
     static_assert(kVecs * kWriters * VEC == kTile, "the writers cover a tile exactly");
-    constexpr int kBufs = MergeShape<ACCUM>::bufs;
+    constexpr int kBufs = Cfg::bufs;
     __shared__ T tiles[kBufs][kTile];
     __shared__ unsigned stage[kMergeWaves][kMsgsPerWave][kRingPairs * PW];  // the rings of chunks, per message
     const int tid = threadIdx.x, lane = tid & 63;
@@ -504,11 +548,28 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
     const unsigned my_tiles = t1 - t0;
     const unsigned steps = my_tiles + (unsigned)kMergeWaves;  // the last tile leaves kMergeWaves steps after it entered
 
-    // headers (the same for every thread)
+    if (!ACCUM && writer) {
+        // every buffer starts as zeros (before anything that waits for memory: the headers are on their way)
+        constexpr int kZeroVecs = kBufs * kTile / VEC;
+        Pack<T, VEC> z;
+#pragma unroll
+        for (int c = 0; c < VEC; ++c) z.x[c] = (T)0;
+        Pack<T, VEC>* const all = reinterpret_cast<Pack<T, VEC>*>(&tiles[0][0]);
+#pragma unroll 4
+        for (int i = tid - 64 * kMergeWaves; i < kZeroVecs; i += kWriters) all[i] = z;
+    }
+    // headers (the same for every thread): both words of all of them in one round trip
+    // (plain loads from addresses that are the same in every lane; an absent message reads `out`)
+    unsigned hdr_n[kMergeMsgs], hdr_k[kMergeMsgs];
+#pragma unroll
+    for (int r = 0; r < kMergeMsgs; ++r) {
+        const unsigned* m = r < n_msgs ? list.msg[r] : reinterpret_cast<const unsigned*>(out);
+        hdr_n[r] = m[0];
+        hdr_k[r] = m[1];
+    }
     bool too_large = false;
 #pragma unroll
-    for (int r = 0; r < kMergeMsgs; ++r)
-        if (r < n_msgs) too_large |= (int)list.msg[r][0] > out_n;
+    for (int r = 0; r < kMergeMsgs; ++r) too_large |= r < n_msgs && (int)hdr_n[r] > out_n;
     if (too_large) {
         if (blockIdx.x == 0 && tid == 0) atomicCAS(&status->code, 0, (int)CX_ERR_MSG_TOO_LARGE);
         if (ACCUM) return;  // add: nothing is touched
@@ -526,8 +587,9 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
     if (loader) {
         // ---- loader wavefronts (accumulating only) ----
         constexpr int kTileDwords = kTile * (int)sizeof(T) / 4;
-        constexpr int kLoadsPerWave = kTileDwords / 64 / kLoaderWaves;  // one dword per lane each
-        static_assert(kLoadsPerWave * 64 * kLoaderWaves == kTileDwords, "the loaders cover a tile exactly");
+        constexpr int kLoadDiv = kLoaderWaves > 0 ? kLoaderWaves : 1;
+        constexpr int kLoadsPerWave = kTileDwords / 64 / kLoadDiv;  // one dword per lane each
+        static_assert(!ACCUM || kLoadsPerWave * 64 * kLoaderWaves == kTileDwords, "the loaders cover a tile exactly");
         const int lw = wave - (kMergeWaves + kWriterWaves);
         const unsigned* const safe = reinterpret_cast<const unsigned*>(out);  // out_n > 0: the first element exists
         auto prefill = [&](unsigned a) {  // tile a of this block: old contents into its buffer
@@ -563,10 +625,6 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
     }
     if (writer) {
         const int wt = tid - 64 * kMergeWaves;
-        if (!ACCUM) {  // every buffer starts as zeros
-            for (int b = 0; b < kBufs; ++b)
-                for (int i = wt; i < kTile; i += kWriters) tiles[b][i] = (T)0;
-        }
         lds_barrier();
         for (unsigned s = 0; s < steps; ++s) {
             const bool draining = s >= (unsigned)kMergeWaves;
@@ -583,8 +641,8 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
                     vec_t vv;
 #pragma unroll
                     for (int c = 0; c < VEC; ++c) vv[c] = v.x[c];
-                    if (CX_MERGE_NT) __builtin_nontemporal_store(vv, reinterpret_cast<vec_t*>(out + base + e));
-                    else *reinterpret_cast<vec_t*>(out + base + e) = vv;
+                    // (nontemporal: the vector is written once; plain stores measured the same)
+                    __builtin_nontemporal_store(vv, reinterpret_cast<vec_t*>(out + base + e));
                 } else if (draining) {
 #pragma unroll
                     for (int c = 0; c < VEC; ++c)
@@ -609,26 +667,32 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
     bool bad = false;
     {
         static_assert(kMsgsPerWave == 1 || kMsgsPerWave == 2, "a wavefront's quarters search two boundaries of up to two messages");
-        unsigned kk[kMsgsPerWave];
+        // search 2s: where the block's range starts in message s, search 2s + 1: where it ends
+        const unsigned* sp[2 * kMsgsPerWave];
+        unsigned sk[2 * kMsgsPerWave], st[2 * kMsgsPerWave], sf[2 * kMsgsPerWave];
 #pragma unroll
         for (int s = 0; s < kMsgsPerWave; ++s) {
             const int r = wave * kMsgsPerWave + s;
-            const unsigned* msg = r < n_msgs ? list.msg[r] : nullptr;
-            const int k = msg ? (int)msg[1] : 0;
-            kk[s] = k > 0 ? (unsigned)k : 0u;
+            const unsigned* msg = nullptr;
+            int k = 0;
+#pragma unroll
+            for (int q = 0; q < kMergeMsgs; ++q)  // (a chain of selects: no indexing of registers)
+                if (q == r && q < n_msgs) {
+                    msg = list.msg[q];
+                    k = (int)hdr_k[q];
+                }
             pairs[s] = msg ? msg + 2 : nullptr;
+            sp[2 * s] = sp[2 * s + 1] = pairs[s];
+            sk[2 * s] = sk[2 * s + 1] = k > 0 ? (unsigned)k : 0u;
+            st[2 * s] = t0 * (unsigned)kTile;  // < 2^31 + tile: fits 32 bits
+            st[2 * s + 1] = t1 * (unsigned)kTile;
         }
-        // quarter 0: start in message 0, quarter 1: end in message 0, quarters 2, 3: message 1
-        const int quarter = lane >> 4;
-        const unsigned* qp = (quarter & 2) ? pairs[kMsgsPerWave - 1] : pairs[0];
-        const unsigned qk = (quarter & 2) ? kk[kMsgsPerWave - 1] : kk[0];
-        const unsigned qt = ((quarter & 1) ? t1 : t0) * (unsigned)kTile;  // < 2^31 + tile: fits 32 bits
-        const unsigned found = quarter_lower_bound<PW>(qp, qk, qt, (unsigned)out_n, lane);
+        wave_lower_bound<PW, 2 * kMsgsPerWave>(sp, sk, st, (unsigned)out_n, lane, reinterpret_cast<const unsigned*>(out + (size_t)t0 * kTile), sf);
 #pragma unroll
         for (int s = 0; s < kMsgsPerWave; ++s) {
             // (wave-uniform values, kept in scalar registers)
-            cur[s] = t0 == 0u ? 0u : (unsigned)__builtin_amdgcn_readlane((int)found, 32 * (s % 2));  // the first block starts at the first pair,
-            end[s] = t1 == ntiles ? kk[s] : (unsigned)__builtin_amdgcn_readlane((int)found, 32 * (s % 2) + 16);  // the last ends behind the last
+            cur[s] = t0 == 0u ? 0u : (unsigned)__builtin_amdgcn_readfirstlane((int)sf[2 * s]);  // the first block starts at the first pair,
+            end[s] = t1 == ntiles ? sk[2 * s] : (unsigned)__builtin_amdgcn_readfirstlane((int)sf[2 * s + 1]);  // the last ends behind the last
             if (end[s] < cur[s]) {  // not sorted
                 bad = true;
                 end[s] = cur[s];
@@ -665,14 +729,20 @@ __global__ __launch_bounds__(MergeShape<ACCUM>::block) void merge_kernel(T* __re
         lane_src[s] = pairs[s] + (size_t)origin[s] * PW + lane;
         ring_base[s] = (unsigned)(uintptr_t)(lptr_t)&stage[wave][s][0];
         if (wave * kMsgsPerWave + s < n_msgs) {
-            // the pair before the slice belongs to the block before: it must lie below this block's range
+            for (unsigned j = 0; j < (unsigned)kRingChunks; ++j) fetch_chunk(s, j);
+            issued[s] = (unsigned)kRingChunks;
+        }
+    }
+    // the pair before the slice belongs to the block before: it must lie below this block's range
+    // (asked for behind the chunks, so that one round trip serves both)
+#pragma unroll
+    for (int s = 0; s < kMsgsPerWave; ++s) {
+        if (wave * kMsgsPerWave + s < n_msgs) {
             unsigned before = kNoPair;
             if (lane == 0 && cur[s] > 0u && cur[s] <= end[s]) before = pairs[s][(size_t)(cur[s] - 1u) * PW];
             before = (unsigned)__builtin_amdgcn_readfirstlane((int)before);
             if (before != kNoPair && before >= t0 * (unsigned)kTile) bad = true;
             last_idx[s] = before;
-            for (unsigned j = 0; j < (unsigned)kRingChunks; ++j) fetch_chunk(s, j);
-            issued[s] = (unsigned)kRingChunks;
         }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the first chunks have landed
@@ -783,33 +853,31 @@ int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_
 template <typename T>
 int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
     if (out_n == 0) return check_headers(h, msgs, n_msgs);
-    constexpr int kTile = MergeTile<T>::value;
-    const unsigned ntiles = (unsigned)(((long long)out_n + kTile - 1) / kTile);
     // persistent blocks: a few per compute unit, each with a contiguous run of tiles
     unsigned want_blocks = (unsigned)(h->cu_count > 0 ? h->cu_count : 256) * (unsigned)h->reduce_blocks_per_cu;
     if (want_blocks < 1u) want_blocks = 1u;
-    unsigned tiles_per_block = (ntiles + want_blocks - 1u) / want_blocks;
-    if (tiles_per_block < 1u) tiles_per_block = 1u;
-    const unsigned grid = (ntiles + tiles_per_block - 1u) / tiles_per_block;
     for (int first = 0; first < n_msgs || first == 0; first += kMergeMsgs) {
         MergeList list;
         const int cnt = n_msgs - first < kMergeMsgs ? n_msgs - first : kMergeMsgs;
         for (int r = 0; r < kMergeMsgs; ++r)
             list.msg[r] = r < cnt ? static_cast<const unsigned*>(msgs[first + r]) : nullptr;
         const bool acc = accumulate || first > 0;
-#define CX_MERGED(OP, ACC)                                                                                        \
-    hipLaunchKernelGGL((merge_kernel<T, OP, ACC>), dim3(grid), dim3(MergeShape<ACC>::block), 0, h->stream, out, out_n, list, \
-                       cnt > 0 ? cnt : 0, ntiles, tiles_per_block, h->d_status)
+#define CX_MERGED(OP, ACC)                                                                                          \
+    do {                                                                                                            \
+        typedef MergeCfg<T, ACC> Cfg;                                                                               \
+        const unsigned ntiles = (unsigned)(((long long)out_n + Cfg::tile - 1) / Cfg::tile);                          \
+        unsigned tiles_per_block = (ntiles + want_blocks - 1u) / want_blocks;                                       \
+        if (tiles_per_block < 1u) tiles_per_block = 1u;                                                             \
+        const unsigned grid = (ntiles + tiles_per_block - 1u) / tiles_per_block;                                    \
+        hipLaunchKernelGGL((merge_kernel<T, OP, ACC>), dim3(grid), dim3(Cfg::block), 0, h->stream, out, out_n, list, \
+                           cnt > 0 ? cnt : 0, ntiles, tiles_per_block, h->d_status);                                \
+    } while (0)
         if (op == 0) {
             CX_MERGED(0, false);
         } else if (!acc) {
             CX_MERGED(1, false);
-        } else if constexpr (sizeof(T) == 4) {
-            CX_MERGED(1, true);
         } else {
-            // 8-byte elements: the rings of 12-byte pairs and seven tiles do not fit one block's LDS
-            int rc = launch_tiled<T>(h, out, out_n, msgs + first, cnt, 1, 1);
-            if (rc != CX_OK) return rc;
+            CX_MERGED(1, true);
         }
 #undef CX_MERGED
         if (n_msgs == 0) break;
@@ -1059,19 +1127,13 @@ int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n
     if (out_n == 0) return check_headers(h, msgs, n_msgs);
     if (mode == 0 && h->reduce_variant == 3) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
     if (mode == 0 && h->reduce_variant == 0) {
-        // Measured on 64 Mi fp32 elements with 1 %-dense messages, 1 / 2 / 4 / 8 messages.  Writing the
-        // vector from zeros: pipelined 53 / 48 / 54 / 63 us against one block per tile 43 / 48 / 62 / 87 us.
-        // Adding into it: pipelined (loader wavefronts) 92 / 92 / 93 / 93 us against 83 / 90 / 110 / 141 us.
-        // With 8-byte elements the accumulating pipeline does not fit a block's LDS.
-        const bool four_bytes = sizeof(T) == 4;
-        if (!accumulate && n_msgs > 1) {
-            if (four_bytes) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, 0);  // later batches of 8 add
-            const int head = n_msgs < kMergeMsgs ? n_msgs : kMergeMsgs;
-            int rc = launch_merged<T>(h, out, out_n, msgs, head, 1, 0);
-            if (rc != CX_OK || head == n_msgs) return rc;
-            return launch_tiled<T>(h, out, out_n, msgs + head, n_msgs - head, 1, 1);
-        }
-        if (accumulate && n_msgs > 2 && four_bytes) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, 1);
+        // Measured on 64 Mi fp32 elements with 1 %-dense messages, 1 / 2 / 3 / 4 / 8 messages (events around
+        // the call).  Writing the vector from zeros: pipelined 61 / 57 / 62 / 62 / 57 us against one block
+        // per tile 45 / 50 / 61 / 66 / 91 us.  Adding into it: pipelined 94 / 100 / 96 / 97 / 94 us against
+        // 87 / 94 / 105 / 114 / 146 us.  32 Mi fp64 elements: from zeros 58 / 57 / 59 / 55 / 63 us against
+        // 43 / 49 / 56 / 62 / 96 us, adding 97 / 101 / 99 / 103 / 97 us against 86 / 95 / 105 / 114 / 155 us.
+        // Later batches of 8 messages add.
+        if (n_msgs > (accumulate ? 2 : 3)) return launch_merged<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
     }
     if (mode == 0 && (h->reduce_variant == 0 || h->reduce_variant == 2))
         return launch_tiled<T>(h, out, out_n, msgs, n_msgs, 1, accumulate);
