@@ -51,6 +51,14 @@ def lib():
         "cx_destroy": (i, [vp]),
         "cx_set_stream": (i, [vp, vp]),
         "cx_synchronize": (i, [vp]),
+        "cx_get_stream": (vp, [vp]),
+        "cx_stream_create": (i, [C.POINTER(vp)]),
+        "cx_stream_destroy": (i, [vp]),
+        "cx_stream_synchronize": (i, [vp]),
+        "cx_event_create": (i, [C.POINTER(vp)]),
+        "cx_event_destroy": (i, [vp]),
+        "cx_event_record": (i, [vp, vp]),
+        "cx_stream_wait_event": (i, [vp, vp]),
         "cx_set_option": (i, [vp, C.c_char_p, i]),
         "cx_profile_read": (i, [vp, C.POINTER(C.c_float), i, C.POINTER(i)]),
         "cx_topk_subsamples": (i, [f, i, f]),

@@ -33,15 +33,23 @@ const char* status_text(int code) {
     }
 }
 
-// Reads and clears the device status word; waits for the stream.
+// Reads and clears the device status; waits for the stream.  `code` holds the first error a kernel
+// recorded; a message cut short for lack of room is noted apart from it (bit 0 of `detail`: the
+// message is valid and error feedback sends the rest later), so that it neither hides a real
+// error nor is hidden by one: a real error is reported first, the note with the next call.
 int collect_status(cx_handle h) {
     CX_HIP(hipMemcpyAsync(h->h_pinned, h->d_status, sizeof(DeviceStatus), hipMemcpyDeviceToHost, h->stream));
     CX_HIP(hipStreamSynchronize(h->stream));
-    const int code = h->h_pinned[0];
+    const int code = h->h_pinned[0], cut_short = h->h_pinned[1] & 1;
     if (code != 0) {
-        CX_HIP(hipMemsetAsync(h->d_status, 0, sizeof(DeviceStatus), h->stream));
+        CX_HIP(hipMemsetAsync(&h->d_status->code, 0, sizeof(int), h->stream));
         CX_HIP(hipStreamSynchronize(h->stream));
         return fail(code, "%s", status_text(code));
+    }
+    if (cut_short) {
+        CX_HIP(hipMemsetAsync(&h->d_status->detail, 0, sizeof(int), h->stream));
+        CX_HIP(hipStreamSynchronize(h->stream));
+        return fail(CX_ERR_CAPACITY, "%s", status_text(CX_ERR_CAPACITY));
     }
     return CX_OK;
 }
@@ -134,6 +142,12 @@ int rle_compress_impl(cx_handle h, void* out_msg, long long out_capacity, const 
 
 template <typename T>
 int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_bytes) {
+    if (h_bytes) {
+        // what earlier calls left behind is reported now, so that the status read below belongs to
+        // this message alone (a message cut short by an earlier compress is not this call's business)
+        const int pending = collect_status(h);
+        if (pending != CX_OK && pending != CX_ERR_CAPACITY) return pending;
+    }
     int rc = launch_decompress<T>(h, static_cast<T*>(out), out_n, msg);
     if (rc != CX_OK || !h_bytes) return rc;
     CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
@@ -283,6 +297,54 @@ int cx_set_stream(cx_handle h, void* hip_stream) {
     return CX_OK;
 }
 
+void* cx_get_stream(cx_handle h) { return h ? static_cast<void*>(h->stream) : nullptr; }
+
+int cx_stream_create(void** out_stream) {
+    if (!out_stream) return fail(CX_ERR_INVALID, "cx_stream_create: null output");
+    *out_stream = nullptr;
+    if (cx_device_count() < 1) return fail(CX_ERR_HIP, "cx_stream_create: no HIP device available");
+    hipStream_t s = nullptr;
+    CX_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
+    *out_stream = static_cast<void*>(s);
+    return CX_OK;
+}
+
+int cx_stream_destroy(void* hip_stream) {
+    if (hip_stream) CX_HIP(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
+    return CX_OK;
+}
+
+int cx_stream_synchronize(void* hip_stream) {
+    CX_HIP(hipStreamSynchronize(static_cast<hipStream_t>(hip_stream)));
+    return CX_OK;
+}
+
+int cx_event_create(void** out_event) {
+    if (!out_event) return fail(CX_ERR_INVALID, "cx_event_create: null output");
+    *out_event = nullptr;
+    hipEvent_t e = nullptr;
+    CX_HIP(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    *out_event = static_cast<void*>(e);
+    return CX_OK;
+}
+
+int cx_event_destroy(void* hip_event) {
+    if (hip_event) CX_HIP(hipEventDestroy(static_cast<hipEvent_t>(hip_event)));
+    return CX_OK;
+}
+
+int cx_event_record(void* hip_event, void* hip_stream) {
+    if (!hip_event) return fail(CX_ERR_INVALID, "cx_event_record: null event");
+    CX_HIP(hipEventRecord(static_cast<hipEvent_t>(hip_event), static_cast<hipStream_t>(hip_stream)));
+    return CX_OK;
+}
+
+int cx_stream_wait_event(void* hip_stream, void* hip_event) {
+    if (!hip_event) return fail(CX_ERR_INVALID, "cx_stream_wait_event: null event");
+    CX_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(hip_stream), static_cast<hipEvent_t>(hip_event), 0));
+    return CX_OK;
+}
+
 int cx_synchronize(cx_handle h) {
     if (!h) return fail(CX_ERR_INVALID, "null handle");
     return collect_status(h);
@@ -377,6 +439,19 @@ int cx_topk_pos(size_t m, float topK) {
         default: return fail(CX_ERR_INVALID, "unknown element type %d", (int)dt); \
     }
 
+// as CX_DISPATCH, but goes on when the call succeeds
+#define CX_DISPATCH_RC(dt, CALL)                                                   \
+    do {                                                                           \
+        int rc__;                                                                  \
+        switch (dt) {                                                              \
+            case CX_F32: { using T = float; rc__ = CALL; break; }                  \
+            case CX_F64: { using T = double; rc__ = CALL; break; }                 \
+            case CX_I32: { using T = int; rc__ = CALL; break; }                    \
+            default: return fail(CX_ERR_INVALID, "unknown element type %d", (int)dt); \
+        }                                                                          \
+        if (rc__ != CX_OK) return rc__;                                            \
+    } while (0)
+
 int cx_topk_threshold(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec, int n, int add_n, float topK,
                       int default_subsamples, float subsample_factor, void* d_thr_out, void* h_thr_out) {
     if (!h || n < 0 || (!vec && n > 0)) return fail(CX_ERR_INVALID, "topk_threshold: bad arguments");
@@ -458,6 +533,11 @@ int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, i
         if (h->h_pinned[8] > out_n)
             return fail(CX_ERR_MSG_TOO_LARGE, "Decompression vector size is bigger than output buffer!");
     }
+    if (check == CX_ADD_ANY_ORDER) {
+        int sorted = 1;
+        CX_DISPATCH_RC(dt, messages_sorted<T>(h, &msg, 1, &sorted));
+        if (!sorted) CX_DISPATCH(dt, launch_sequential<T>(h, static_cast<T*>(out), out_n, msg, 1));
+    }
     CX_DISPATCH(dt, launch_add<T>(h, static_cast<T*>(out), out_n, msg, 0));
 }
 
@@ -467,6 +547,18 @@ int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* con
     for (int r = 0; r < n_msgs; ++r)
         if (!msgs || !msgs[r] || !aligned4(msgs[r]))
             return fail(CX_ERR_INVALID, "message %d must be a 4-byte aligned device pointer", r);
+    if ((mode & CX_REDUCE_ANY_ORDER) && n_msgs > 0) {
+        int sorted = 1;
+        CX_DISPATCH_RC(dt, messages_sorted<T>(h, msgs, n_msgs, &sorted));
+        if (!sorted) {
+            // the reference's loop, message after message, pair after pair (src/compressor.hxx:640-658)
+            if (!accumulate) CX_DISPATCH_RC(dt, launch_zero<T>(h, static_cast<T*>(out), out_n));
+            for (int r = 0; r < n_msgs; ++r)
+                CX_DISPATCH_RC(dt, launch_sequential<T>(h, static_cast<T*>(out), out_n, msgs[r], 1));
+            return CX_OK;
+        }
+    }
+    mode &= ~CX_REDUCE_ANY_ORDER;
     CX_DISPATCH(dt, launch_reduce<T>(h, static_cast<T*>(out), out_n, msgs, n_msgs, accumulate, mode));
 }
 

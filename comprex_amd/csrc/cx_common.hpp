@@ -70,7 +70,8 @@ struct SelectState {
     PickState pass_state[kMaxRadixPasses];
 };
 
-// Device status word: first error wins.
+// Device status: `code` = the first error a kernel recorded (first wins); bit 0 of `detail` = a
+// compressed message was cut short for lack of room (not an error of the message: see collect_status).
 struct DeviceStatus {
     int code;
     int detail;
@@ -174,6 +175,8 @@ template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, cons
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);
 // the reference's loop, pair after pair: any index order, indices repeated anywhere (slow)
 template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, const void* msg, int add);
+// one pass over the messages' indices and one wait: *sorted = every message's indices ascend
+template <typename T> int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted);
 template <typename T>
 int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode);
 int launch_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity);

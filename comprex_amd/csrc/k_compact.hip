@@ -250,7 +250,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
             }
         }
     }
-    if (DIRECT && overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    if (DIRECT && overflow) atomicOr(&status->detail, 1);
     return total;
 }
 
@@ -427,7 +427,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
                 }
             }
     }
-    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    if (overflow) atomicOr(&status->detail, 1);
 
     if (inline_redo && deferred != 0ull) {
         const T thr = thr_ptr ? *thr_ptr : thr_val;
@@ -789,7 +789,7 @@ __global__ __launch_bounds__(kFilterBlock) void filter_write_kernel(
         pos += all;
         __syncthreads();
     }
-    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    if (overflow) atomicOr(&status->detail, 1);
     if (blockIdx.x == kFilterBlocks - 1 && tid == 0) {
         if ((long long)pos > cap_pairs) pos = (unsigned)cap_pairs;  // never announce more than was written
         msg_words[0] = (unsigned)n;

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kBlock) void rle_write_kernel(const unsigned* __res
             const int bytes = 16 + 4 * (int)runs;
             if (size_prefix) *size_prefix = bytes;
             result[0] = bytes;
-            if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+            if (overflow) atomicOr(&status->detail, 1);
         }
         return;
     }
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kBlock) void rle_write_kernel(const unsigned* __res
         }
         runs_before += chunk_total;
     }
-    if (overflow) atomicCAS(&status->code, 0, (int)CX_ERR_CAPACITY);
+    if (overflow) atomicOr(&status->detail, 1);
 }
 
 // A message that did not fit (result[0] = its true size > capacity): nothing of it may be taken

@@ -62,6 +62,7 @@ __global__ __launch_bounds__(kBlock) void scatter_kernel(T* __restrict__ out, in
         if (OP == 2) {
             atomic_accumulate(out + idx, load_value<T>(p + 1));
         } else if (OP == 1) {
+            if (j > 0 && (unsigned)p[-PW] > (unsigned)idx) bad = true;  // not index-sorted: equal indices may lie apart
             if (j > 0 && (int)p[-PW] == idx) continue;  // not the head of its run
             T acc = out[idx];
             long long q = j;
@@ -125,6 +126,20 @@ __global__ __launch_bounds__(64) void sequential_kernel(T* out, int out_n,
         __threadfence_block();
     }
     if (bad) atomicCAS(&status->code, 0, (int)CX_ERR_INDEX);
+}
+
+// *unsorted |= some message holds an index below its predecessor (or is made for a longer vector,
+// which the caller's path then reports).  grid.y = message.  The fast paths need ascending indices;
+// a caller that must take any order (the reference's loops do) asks first.
+__global__ __launch_bounds__(kBlock) void order_check_kernel(MsgHeaders list, unsigned* __restrict__ unsorted, int pair_words) {
+    const unsigned* msg = list.msg[blockIdx.y];
+    const long long k = (long long)(int)msg[1];
+    const unsigned* pairs = msg + 2;
+    const long long stride = (long long)gridDim.x * kBlock;
+    bool bad = false;
+    for (long long j = (long long)blockIdx.x * kBlock + threadIdx.x + 1; j < k; j += stride)
+        bad |= pairs[(size_t)pair_words * j] < pairs[(size_t)pair_words * (j - 1)];
+    if (__any(bad) && (threadIdx.x & 63) == 0) atomicOr(unsorted, 1u);
 }
 
 // ---- tiled, rank-ordered reduce ------------------------------------------------------------
@@ -1091,6 +1106,28 @@ template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, cons
     return CX_OK;
 }
 
+// Are all the messages index-sorted?  One pass over their indices and one wait for the stream.
+template <typename T> int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted) {
+    *sorted = 1;
+    unsigned* flag = reinterpret_cast<unsigned*>(h->d_status) + 16;  // a word of the status block
+    for (int first = 0; first < n_msgs; first += MsgHeaders::kMax) {
+        MsgHeaders list;
+        const int cnt = n_msgs - first < MsgHeaders::kMax ? n_msgs - first : MsgHeaders::kMax;
+        for (int r = 0; r < MsgHeaders::kMax; ++r)
+            list.msg[r] = r < cnt ? static_cast<const unsigned*>(msgs[first + r]) : nullptr;
+        hipLaunchKernelGGL(order_check_kernel, dim3(256, cnt), dim3(kBlock), 0, h->stream, list, flag,
+                           (int)Elem<T>::pair_words);
+    }
+    CX_HIP(hipGetLastError());
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 13, flag, sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
+    CX_HIP(hipStreamSynchronize(h->stream));
+    if (h->h_pinned[13] != 0) {
+        *sorted = 0;
+        CX_HIP(hipMemsetAsync(flag, 0, sizeof(unsigned), h->stream));
+    }
+    return CX_OK;
+}
+
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic) {
     if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "add: bad arguments");
     if (out_n == 0) return check_headers(h, &msg, 1);
@@ -1163,6 +1200,7 @@ template int reserve_reduce<int>(cx_handle, int);
     template int launch_threshold_apply<T>(cx_handle, T*, T*, const T*, int, const T*, const T*); \
     template int launch_add<T>(cx_handle, T*, int, const void*, int);                             \
     template int launch_sequential<T>(cx_handle, T*, int, const void*, int);                      \
+    template int messages_sorted<T>(cx_handle, const void* const*, int, int*);                    \
     template int launch_decompress<T>(cx_handle, T*, int, const void*);                           \
     template int launch_reduce<T>(cx_handle, T*, int, const void* const*, int, int, int);
 CX_INSTANTIATE(float)

@@ -115,17 +115,32 @@ public:
     // fixes the order of the floating-point additions, as the loop does) by one rank-ordered reduce.
     void reduce_workers(data_t* data, int size) {
         const int numRanks = this->gaspi_env->get_ranks();
-        std::vector<const void*> messages;
         int first = -1;
+        for (int rank = 0; rank < numRanks && first < 0; ++rank)
+            if (rank != chiefRank) first = rank;
+        if (first < 0) return;
+        FastComprEx<data_t>* reader = &comm_reduce_map[first];  // its stream reads every message
+        // every channel whose message was taken is released when this call leaves, also by an exception
+        struct Taken {
+            std::vector<FastComprEx<data_t>*> from;
+            FastComprEx<data_t>* reader;
+            ~Taken() {
+                for (auto* c : from) {
+                    try {
+                        c->message_done(reader);
+                    } catch (...) {
+                    }
+                }
+            }
+        } taken;
+        taken.reader = reader;
+        std::vector<const void*> messages;
         for (int rank = 0; rank < numRanks; ++rank) {
             if (rank == chiefRank) continue;
-            messages.push_back(comm_reduce_map[rank].waiting_message());
-            if (first < 0) first = rank;
+            messages.push_back(comm_reduce_map[rank].waiting_message(reader));
+            taken.from.push_back(&comm_reduce_map[rank]);
         }
-        if (first < 0) return;
-        comm_reduce_map[first].add_messages(data, size, messages.data(), (int)messages.size());
-        for (int rank = 0; rank < numRanks; ++rank)
-            if (rank != chiefRank) comm_reduce_map[rank].message_done();
+        reader->add_messages(data, size, messages.data(), (int)messages.size());
     }
 
     void reset() {

@@ -7,7 +7,11 @@
 //   * the residual ("rests") lives in device memory, and so do the send/receive buffers;
 //   * the GaspiCxx Source/TargetBuffer pair is replaced by one device buffer per directed
 //     (source, target, tag) triple, owned by the GaspiEnvironment stand-in: the sender's
-//     compressor writes the message where the receiver reads it, ordered by the HIP stream;
+//     compressor writes the message where the receiver reads it.  Every object works on a HIP
+//     stream of its own (shared with its compressor and threshold clones); a message's
+//     hand-over is an event the sender's stream records and the receiver's stream waits for,
+//     and every call joins the object's stream with the caller's (GaspiEnvironment::
+//     set_user_stream, default the null stream) on entry and on exit;
 //   * `vector` arguments may be host pointers (staged) or device pointers (used in place);
 //   * with one thread playing all ranks a receive with no message pending throws instead of
 //     blocking for ever; with one thread per rank (GaspiEnvironment::set_blocking) it waits;
@@ -49,10 +53,23 @@ protected:
     cxx::Handle handle_;
     cxx::DeviceBuffer stage_;
     cxx::DeviceBuffer forward_;  // message in transit between inbox and outbox (forward_buffer)
+    cxx::StreamOrder cross_;     // for the calls that touch another object's buffers
 
     VarTYPE* rests() const { return static_cast<VarTYPE*>(restsVect.data()); }
     char* src_address() const { return static_cast<char*>(srcBuff_data->buffer.data()); }
     char* targ_address() const { return static_cast<char*>(targBuff_data->buffer.data()); }
+
+    // this object's stream (its compressor and threshold clones work on it too)
+    void* stream() { return handle_.ctx().stream(); }
+    // joins the object's stream with the caller's for the time of a call
+    cxx::StreamCtx& joined() {
+        handle_.ctx().set_origin(gaspiCxx_segment ? gaspiCxx_segment->user_stream() : nullptr);
+        return handle_.ctx();
+    }
+    void bind_clones() {
+        compressor->bind_stream(handle_.ctx_ptr());
+        threshold->bind_stream(handle_.ctx_ptr());
+    }
 
     void alloc_rests() {
         restsVect.reserve((size_t)size * sizeof(VarTYPE));
@@ -62,11 +79,11 @@ protected:
 
     // "waitForCompletion" of the reference's TargetBuffer
     void wait_for_message() {
-        targBuff_data->wait_message(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s());
+        targBuff_data->wait_message(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s(), stream());
     }
     // the source buffer may be overwritten once the receiver has read the previous message
     void wait_for_room() {
-        srcBuff_data->wait_consumed(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s());
+        srcBuff_data->wait_consumed(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s(), stream());
     }
 
     // send-side tail shared by all write paths: data-only / update-only / fused compression
@@ -112,7 +129,9 @@ protected:
 public:
     ComprEx()
         : compressor(new CompressorNone<VarTYPE>()), threshold(new ThresholdNone<VarTYPE>()), gaspiCxx_segment(NULL),
-          rests_size(0), srcRank(-1), targRank(-1), size(0), bufferSize(0), size_factor(0), send_sizeBytes(false) {}
+          rests_size(0), srcRank(-1), targRank(-1), size(0), bufferSize(0), size_factor(0), send_sizeBytes(false) {
+        bind_clones();
+    }
 
     ComprEx(GaspiEnvironment* segment, int size, float size_factor = 1.0, bool send_sizeBytes = false)
         : compressor(new CompressorNone<VarTYPE>()), threshold(new ThresholdNone<VarTYPE>()),
@@ -120,6 +139,7 @@ public:
           send_sizeBytes(send_sizeBytes) {
         // the reference evaluates size*sizeof(T)*size_factor in fp32 and truncates to int; 64 bits here
         bufferSize = (long long)((float)((size_t)size * sizeof(VarTYPE)) * size_factor);
+        bind_clones();
     }
 
     virtual ~ComprEx() {}
@@ -132,6 +152,7 @@ public:
         gaspiCxx_segment = other.gaspiCxx_segment;
         compressor.reset(other.compressor->clone());
         threshold.reset(other.threshold->clone());
+        bind_clones();
         size = other.size;
         bufferSize = other.bufferSize;
         size_factor = other.size_factor;
@@ -143,17 +164,30 @@ public:
         } else {
             rests_size = 0;
         }
+        reserve_scratch();  // the clones' scratch too: the exchange calls never allocate
         return *this;
     }
+
+    // Not in the reference: run this object's GPU work (its clones' included) on a stream of the
+    // caller's instead of its own (NULL = the null stream).  Waits for what the old stream holds.
+    void set_stream(void* hip_stream) {
+        handle_.ctx().adopt(hip_stream);
+        handle_.refresh();
+        compressor->stream_changed();
+        threshold->stream_changed();
+    }
+    void* get_stream() { return stream(); }
 
     void setCompressor(const Compressor<VarTYPE>& c) { setCompressor(&c); }
     void setCompressor(const Compressor<VarTYPE>* c) {
         this->compressor.reset(c->clone());
+        bind_clones();
         reserve_scratch();
     }
     void setThreshold(const ThresholdFunction<VarTYPE>& t) { setThreshold(&t); }
     void setThreshold(const ThresholdFunction<VarTYPE>* t) {
         this->threshold.reset(t->clone());
+        bind_clones();
         reserve_scratch();
     }
 
@@ -173,7 +207,7 @@ public:
 
     virtual void resetRests() {
         if (rests_size > 0)
-            cxx::check(cx_zero(handle_.get(), cxx::dtype_of<VarTYPE>::value, rests(), rests_size));
+            cxx::check(cx_zero(handle_.get(), cxx::dtype_of<VarTYPE>::value, rests(), rests_size));  // (own memory, own stream)
     }
 
     // Sends the whole residual (no thresholding: every non-zero element) and clears it.
@@ -185,7 +219,7 @@ public:
         // compresses the residual as data and clears it afterwards: the same message and residual)
         compress_into(0, nullptr, rests(), rests_size, false);
         const int st = compressor->device_status();
-        srcBuff_data->post();
+        srcBuff_data->post(stream());
         report_flush(st);
         resetRests();
     }
@@ -207,6 +241,7 @@ public:
                      rests_size);
             throw std::runtime_error(error_msg);
         }
+        cxx::Scope scope(const_cast<ComprEx<VarTYPE>*>(this)->joined());
         cx_handle h = const_cast<ComprEx<VarTYPE>*>(this)->handle_.get();
         cxx::check(cx_copy(h, data, rests(), (size_t)size * sizeof(VarTYPE)));
         cxx::check(cx_synchronize(h));
@@ -220,6 +255,7 @@ public:
             throw std::runtime_error(error_msg);
         }
         ComprEx<VarTYPE>* self = const_cast<ComprEx<VarTYPE>*>(this);
+        cxx::Scope scope(self->joined());
         cx_handle h = self->handle_.get();
         cxx::Staged<VarTYPE> d(h, self->stage_, data, (size_t)size, true, true);
         cxx::check(cx_add_vec(h, cxx::dtype_of<VarTYPE>::value, d.get(), rests(), size));
@@ -239,6 +275,7 @@ public:
     // residual += vector; entries above the threshold are sent and cleared
     virtual void writeRemote(const VarTYPE* vector, int size) {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cxx::Scope scope(joined());
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
         float topK = 0;
@@ -247,7 +284,7 @@ public:
             const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
             if (fused_topk_into(src_address() + offset, bufferSize - offset, v.get(), size,
                                 send_sizeBytes ? reinterpret_cast<int*>(src_address()) : nullptr)) {
-                srcBuff_data->post();
+                srcBuff_data->post(stream());
                 return;
             }
         }
@@ -260,63 +297,85 @@ public:
         }
         wait_for_room();
         compress_into(0, v.get(), rests(), rests_size, true);
-        srcBuff_data->post();
+        srcBuff_data->post(stream());
     }
 
     // compression only: no threshold, residual untouched
     virtual void writeRemote_compressOnly(const VarTYPE* vector, int size) {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cxx::Scope scope(joined());
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
         wait_for_room();
         compress_into(0, v.get(), nullptr, size, false);
-        srcBuff_data->post();
+        srcBuff_data->post(stream());
     }
 
     // threshold from the vector alone, residual untouched
     void writeRemote_NoResidual(const VarTYPE* vector, int size) {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
+        cxx::Scope scope(joined());
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
         threshold->prepare(v.get(), size);
         wait_for_room();
         compress_into(0, v.get(), nullptr, size, true);
-        srcBuff_data->post();
+        srcBuff_data->post(stream());
     }
 
     // overwrites `vector` with the received message
     virtual void readRemote(VarTYPE* vector, int size) {
         if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
+        cxx::Scope scope(joined());
         wait_for_message();
+        Release release(this);  // the channel is freed whatever the decoder reports
         const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
         compressor->decompress(vector, size, targ_address() + offset);
-        targBuff_data->consumed();
     }
 
     // adds the received message to `vector`
     virtual void readRemote_add(VarTYPE* vector, int size) {
         if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
+        cxx::Scope scope(joined());
         wait_for_message();
+        Release release(this);
         const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
         compressor->add(vector, size, targ_address() + offset);
-        targBuff_data->consumed();
     }
 
+protected:
+    // marks the pending message consumed when the receive leaves, also by an exception
+    struct Release {
+        ComprEx* c;
+        explicit Release(ComprEx* c) : c(c) {}
+        ~Release() {
+            try {
+                c->targBuff_data->consumed(c->stream());
+            } catch (...) {
+            }
+        }
+    };
+
+public:
     // Not in the reference: a receiver that takes the messages of several channels in one call (the
     // chief of the all-to-one schedule) waits for each, collects their device addresses, adds them all
     // with add_messages() of one of the objects, and releases the channels with message_done().
-    const void* waiting_message() {
+    // `reader`: the object whose add_messages() will read the message (its stream waits for it)
+    const void* waiting_message(ComprEx<VarTYPE>* reader = nullptr) {
         if (!targBuff_data) throw std::runtime_error("Receive issued without connecting to Remote!");
-        wait_for_message();
+        targBuff_data->wait_message(gaspiCxx_segment->blocking(), gaspiCxx_segment->timeout_s(),
+                                    (reader ? reader : this)->stream());
         return targ_address() + (send_sizeBytes ? (int)sizeof(int) : 0);
     }
-    void message_done() { targBuff_data->consumed(); }
+    void message_done(ComprEx<VarTYPE>* reader = nullptr) { targBuff_data->consumed((reader ? reader : this)->stream()); }
     void add_messages(VarTYPE* vector, int size, const void* const* messages, int count) {
+        cxx::Scope scope(joined());
         compressor->add_many(vector, size, messages, count);
     }
 
     // receive, pass the compressed message on to this object's target, and decompress it
     void readRemote_forward(VarTYPE* vector, int size) {
+        cxx::Scope scope(joined());
         wait_for_message();
         wait_for_room();
         cx_handle h = handle_.get();
@@ -324,14 +383,14 @@ public:
             int sizeBytes = 0;
             cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
             cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
-            srcBuff_data->post();
+            srcBuff_data->post(stream());
             compressor->decompress(vector, size, targ_address() + sizeof(int));
         } else {
             const int sizeBytes = compressor->decompress(vector, size, targ_address());
             cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes));
-            srcBuff_data->post();
+            srcBuff_data->post(stream());
         }
-        targBuff_data->consumed();
+        targBuff_data->consumed(stream());
     }
 
     void readRemote_forwardCopy(VarTYPE* vector, int size) {
@@ -343,7 +402,7 @@ public:
         int sizeBytes = 0;
         cxx::check(cx_copy(h, &sizeBytes, targ_address(), sizeof(int)));
         cxx::check(cx_copy(h, src_address(), targ_address(), (size_t)sizeBytes + sizeof(int)));
-        targBuff_data->consumed();
+        targBuff_data->consumed(stream());
     }
 
     void readRemote_wait() { wait_for_message(); }
@@ -360,7 +419,7 @@ public:
         const size_t bytes = (size_t)sizeBytes + sizeof(int);
         void* hold = forward_.reserve(bytes);
         cxx::check(cx_copy(h, hold, targ_address(), bytes));
-        targBuff_data->consumed();
+        targBuff_data->consumed(stream());
         wait_for_room();
         cxx::check(cx_copy(h, src_address(), hold, bytes));
     }
@@ -368,8 +427,9 @@ public:
     // sends the message sitting in the send buffer and adds it to `vector`
     void forward_add(VarTYPE* vector, int size) {
         if (!this->send_sizeBytes) throw std::runtime_error("If using forward_add, send_sizeBytes must be true!");
+        cxx::Scope scope(joined());
         compressor->add(vector, size, src_address() + sizeof(int));
-        srcBuff_data->post();
+        srcBuff_data->post(stream());
     }
 
     virtual void connectTx(int targRank, int tag) {
@@ -436,7 +496,7 @@ protected:
         this->wait_for_room();
         const long long room = doublebuffer_offset < this->bufferSize ? doublebuffer_offset : this->bufferSize;
         cxx::check(cx_copy_counted(h, this->src_address(), half(off), half_bytes(off), room));
-        srcBuff_data->post();
+        srcBuff_data->post(this->stream());
     }
 
     void compress_half(long long off, const VarTYPE* d_data, VarTYPE* d_update, int n, bool use_threshold) {
@@ -466,6 +526,12 @@ public:
         return *this;
     }
 
+    // the halves are taken when the object connects: the exchange calls never allocate
+    virtual void connectTx(int targRank, int tag) {
+        ComprEx<VarTYPE>::connectTx(targRank, tag);
+        ensure_halves();
+    }
+
     virtual void flushRests() {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         ensure_halves();
@@ -492,6 +558,7 @@ public:
     virtual void writeRemote(const VarTYPE* vector, int size) {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         ensure_halves();
+        cxx::Scope scope(this->joined());
         cx_handle h = this->handle_.get();
         const long long wo = write_offset(), so = send_offset();
         if (is_first) {
@@ -519,6 +586,7 @@ public:
     virtual void writeRemote_compressOnly(VarTYPE* vector, int size) {
         if (!srcBuff_data) throw std::runtime_error("Send issued without connecting to Remote!");
         ensure_halves();
+        cxx::Scope scope(this->joined());
         cx_handle h = this->handle_.get();
         const long long wo = write_offset(), so = send_offset();
         if (is_first) {
@@ -545,12 +613,17 @@ public:
         }
         send_half(so);
         if (!other->is_first) {
-            // memcpy(..., other->sizeBytes) and sizeBytes = other->sizeBytes, both on the device
+            // memcpy(..., other->sizeBytes) and sizeBytes = other->sizeBytes, both on the device.  The
+            // other object compressed on ITS stream: this one's waits for that, and the other's next
+            // compress into the same half waits for this copy.
+            FastComprEx* src = const_cast<FastComprEx*>(other);
             const long long oso = other->send_offset();
-            const long long room = doublebuffer_offset < other->doublebuffer_offset ? doublebuffer_offset
-                                                                                  : other->doublebuffer_offset;
-            cxx::check(cx_copy_counted(h, half(wo), other->half(oso), other->half_bytes(oso), room));
+            if (other->doublebuffer_offset > doublebuffer_offset)
+                throw std::runtime_error("writeRemote_sameAs: this object's buffer is smaller than the other's!");
+            this->cross_.order(src->stream(), this->stream());
+            cxx::check(cx_copy_counted(h, half(wo), other->half(oso), other->half_bytes(oso), doublebuffer_offset));
             cxx::check(cx_copy(h, half_bytes(wo), other->half_bytes(oso), sizeof(int)));
+            this->cross_.order(this->stream(), src->stream());
         } else {
             this->is_first = true;
         }

@@ -17,6 +17,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <memory>
 #include <stdexcept>
 
 #include "cx_device.hxx"
@@ -32,23 +33,28 @@ public:
     // writes the compressed vector into targetBuffer, returns the bytes written
     virtual int compress(void* targetBuffer, const VarTYPE* data_vector, const int data_vector_size,
                          VarTYPE threshold) {
+        cxx::Scope scope(handle_.ctx());
         return compression_strategy(targetBuffer, data_vector, NULL, data_vector_size, threshold);
     }
     virtual int compress_update(void* targetBuffer, VarTYPE* update_vector, const int update_vector_size,
                                 VarTYPE threshold) {
+        cxx::Scope scope(handle_.ctx());
         return compression_strategy(targetBuffer, NULL, update_vector, update_vector_size, threshold);
     }
     virtual int compress_add_update(void* targetBuffer, VarTYPE* update_vector, const int update_vector_size,
                                     const VarTYPE* data_vector, const int data_vector_size, VarTYPE threshold) {
         check_sizes(update_vector_size, data_vector_size);
+        cxx::Scope scope(handle_.ctx());
         return compression_strategy(targetBuffer, data_vector, update_vector, update_vector_size, threshold);
     }
 
     // returns the bytes consumed from sourceBuffer
     virtual int decompress(VarTYPE* output, int output_size, const void* sourceBuffer) {
+        cxx::Scope scope(handle_.ctx());
         return decompression_strategy(output, output_size, sourceBuffer);
     }
     virtual void add(VarTYPE* output, int output_size, const void* sourceBuffer) {
+        cxx::Scope scope(handle_.ctx());
         return add_strategy(output, output_size, sourceBuffer);
     }
 
@@ -60,6 +66,12 @@ public:
     virtual void add_many(VarTYPE* output, int output_size, const void* const* d_sources, int count) {
         for (int i = 0; i < count; ++i) add(output, output_size, d_sources[i]);
     }
+
+    // Not in the reference: the stream this object's GPU work runs on and the caller's stream it is
+    // joined with around every call (cx_device.hxx).  A ComprEx binds its clones to its own.
+    void bind_stream(const std::shared_ptr<cxx::StreamCtx>& ctx) { handle_.bind(ctx); }
+    cxx::StreamCtx& stream_context() { return handle_.ctx(); }
+    void stream_changed() { handle_.refresh(); }
 
     // Not in the reference: bytes of the largest message a vector of n elements can produce.
     virtual long long max_message_bytes(int n) const = 0;
@@ -100,6 +112,13 @@ protected:
                                      const int vector_size, VarTYPE threshold) = 0;
     virtual int decompression_strategy(VarTYPE* output, int output_size, const void* input) = 0;
     virtual void add_strategy(VarTYPE* output, int output_size, const void* sourceBuffer) = 0;
+
+    // Status of a receive: a message that an earlier SEND of this compressor had to cut short is no
+    // concern of the receive (the note is dropped; flushRests sends what stayed behind).
+    static int receive_status(cx_handle h) {
+        const int rc = cx_synchronize(h);
+        return rc == CX_ERR_CAPACITY ? cx_synchronize(h) : rc;
+    }
 
     static void check_sizes(int update_vector_size, int data_vector_size) {
         if (data_vector_size != update_vector_size) {
@@ -213,8 +232,9 @@ protected:
         cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
         // the kernel reads the header itself: a message made for a longer vector touches nothing and
         // is reported by the one wait below (the reference throws before it touches the output)
-        cxx::check(cx_ip_add(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_in, 0));
-        const int rc = cx_synchronize(h);
+        // (any index order, as the reference takes: the call looks at the indices first)
+        int rc = cx_ip_add(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_in, CX_ADD_ANY_ORDER);
+        if (rc == CX_OK) rc = Compressor<VarTYPE>::receive_status(h);
         if (rc == CX_ERR_MSG_TOO_LARGE)
             throw std::runtime_error("Decompression vector size is bigger than output buffer!");
         cxx::check(rc);
@@ -228,10 +248,12 @@ public:
     // `output` untouched.
     virtual void add_many(VarTYPE* output, int output_size, const void* const* d_sources, int count) {
         if (count <= 0) return;
+        cxx::Scope scope(this->handle_.ctx());
         cx_handle h = this->handle_.get();
         cxx::Staged<VarTYPE> o(h, this->stage_a_, output, (size_t)output_size, true, true);
-        cxx::check(cx_ip_reduce(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_sources, count, 1, 0));
-        const int rc = cx_synchronize(h);
+        cxx::check(cx_ip_reduce(h, cxx::dtype_of<VarTYPE>::value, o.get(), output_size, d_sources, count, 1,
+                                CX_REDUCE_ANY_ORDER));
+        const int rc = Compressor<VarTYPE>::receive_status(h);
         if (rc == CX_ERR_MSG_TOO_LARGE)
             throw std::runtime_error("Decompression vector size is bigger than output buffer!");
         cxx::check(rc);

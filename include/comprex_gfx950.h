@@ -96,6 +96,21 @@ int cx_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes,
 int cx_create(cx_handle* out, void* hip_stream /* hipStream_t, NULL = default stream */);
 int cx_destroy(cx_handle h);
 int cx_set_stream(cx_handle h, void* hip_stream);
+void* cx_get_stream(cx_handle h);
+
+/* Streams and events for callers that hold no HIP headers (the C++ classes of include/ (.hxx) are
+ * plain host code).  The reference's RDMA put is asynchronous and its receiver waits for a
+ * notification (src/comprEx.tpp:190,231,243): here every ComprEx object works on a stream of its
+ * own and a message's hand-over is an event the sender records and the receiver's stream waits
+ * for.  Streams are created non-blocking (no implicit ordering with the null stream) and at the
+ * default priority; events carry no timing.  A NULL stream argument names the null stream. */
+int cx_stream_create(void** out_stream);
+int cx_stream_destroy(void* hip_stream);
+int cx_stream_synchronize(void* hip_stream);
+int cx_event_create(void** out_event);
+int cx_event_destroy(void* hip_event);
+int cx_event_record(void* hip_event, void* hip_stream);
+int cx_stream_wait_event(void* hip_stream, void* hip_event);
 /* Waits for the handle's stream and returns the first device-side error seen since the
  * last call (CX_OK if none), clearing it. */
 int cx_synchronize(cx_handle h);
@@ -221,7 +236,13 @@ int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void*
 /* CompressorIndexPairs<T>::add_strategy (src/compressor.hxx:640-658): out[index] += value
  * in message order.  A message whose n exceeds out_n changes nothing and records
  * CX_ERR_MSG_TOO_LARGE.  `check` != 0 reads the header first and returns that error
- * synchronously, as the reference throws before touching `out`. */
+ * synchronously, as the reference throws before touching `out`.
+ * Index order: the kernel applies a run of equal NEIGHBOURING indices in message order, which is
+ * all an index-sorted message (what the compressors emit) needs; an index below its predecessor
+ * records CX_ERR_INDEX, because equal indices may then lie apart and `out` is no longer what the
+ * reference's loop gives.  check == CX_ADD_ANY_ORDER looks at the indices first (one pass, one more
+ * wait) and applies a message that is not sorted pair after pair, exactly as the reference does. */
+enum { CX_ADD_ANY_ORDER = 2 };
 int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int check);
 
 /* The chief's reduce loop of Comprex_AllToOneAllreduce::apply (src/allreduce.tpp:183-189):
@@ -232,7 +253,11 @@ int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, i
  * neighbours); mode 1 = one launch of floating-point atomics per message, in the order given:
  * the additions to an element are reordered only among pairs of ONE message that share its
  * index.  An empty `out` (out_n == 0) writes nothing and still refuses messages made for a
- * longer vector (CX_ERR_MSG_TOO_LARGE). */
+ * longer vector (CX_ERR_MSG_TOO_LARGE).  mode | CX_REDUCE_ANY_ORDER: the call first looks at the
+ * indices (one pass, one wait for the stream) and, when a message is not index-sorted, applies the
+ * messages one after the other, pair after pair, as the reference's loop does: any order, equal
+ * indices anywhere; without it such a message records CX_ERR_INDEX and leaves `out` undefined. */
+enum { CX_REDUCE_ANY_ORDER = 4 };
 int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* const* msgs, int n_msgs,
                  int accumulate, int mode);
 

@@ -10,6 +10,7 @@
 #define CX_DEVICE_HXX
 
 #include <cstddef>
+#include <memory>
 #include <stdexcept>
 #include <string>
 #include <type_traits>
@@ -27,19 +28,134 @@ template <> struct dtype_of<float> { static constexpr cx_dtype value = CX_F32; }
 template <> struct dtype_of<double> { static constexpr cx_dtype value = CX_F64; };
 template <> struct dtype_of<int> { static constexpr cx_dtype value = CX_I32; };
 
-// One handle (stream + scratch) per object, created on first use so that constructing and
-// cloning threshold/compressor objects never touches the GPU.
+// The stream an object's GPU work runs on, and the stream its caller's vectors live on.
+//
+// The reference's calls are synchronous host code; here they enqueue GPU work.  Every object
+// (a ComprEx with its compressor and threshold clones, or a compressor / threshold used on its
+// own) has a stream of its own, so that independent channels overlap and nothing depends on the
+// null stream.  What keeps a caller's vector safe is a pair of joins around every call that
+// touches it: on entry the object's stream waits for the work the caller's stream ("origin",
+// NULL = the null stream, where plain hipMemcpy / framework default-stream work runs) has been
+// given so far, on exit the origin waits for the object's stream.  Both are events: the host
+// never blocks.  Scopes nest (a ComprEx call that runs its threshold's prepare joins once).
+class StreamCtx {
+public:
+    StreamCtx() : stream_(nullptr), owned_(false), made_(false), origin_(nullptr), ev_(nullptr), depth_(0) {}
+    StreamCtx(const StreamCtx&) = delete;
+    StreamCtx& operator=(const StreamCtx&) = delete;
+    ~StreamCtx() {
+        if (ev_) cx_event_destroy(ev_);
+        if (owned_ && stream_) {
+            cx_stream_synchronize(stream_);
+            cx_stream_destroy(stream_);
+        }
+    }
+    // the object's stream, created on first use
+    void* stream() {
+        if (!made_) {
+            check(cx_stream_create(&stream_));
+            owned_ = true;
+            made_ = true;
+        }
+        return stream_;
+    }
+    // run on a stream of the caller's instead (not owned; NULL = the null stream)
+    void adopt(void* hip_stream) {
+        if (made_ && owned_ && stream_) {
+            check(cx_stream_synchronize(stream_));
+            check(cx_stream_destroy(stream_));
+        }
+        stream_ = hip_stream;
+        owned_ = false;
+        made_ = true;
+    }
+    void set_origin(void* hip_stream) { origin_ = hip_stream; }
+    void* origin() const { return origin_; }
+
+    void enter() {
+        if (depth_++ > 0) return;
+        void* s = stream();
+        if (s == origin_) return;
+        check(cx_event_record(event(), origin_));
+        check(cx_stream_wait_event(s, event()));
+    }
+    void leave() {
+        if (--depth_ > 0) return;
+        void* s = stream();
+        if (s == origin_) return;
+        if (cx_event_record(event(), s) == CX_OK) cx_stream_wait_event(origin_, event());
+    }
+
+private:
+    void* event() {
+        if (!ev_) check(cx_event_create(&ev_));
+        return ev_;
+    }
+    void* stream_;
+    bool owned_, made_;
+    void* origin_;
+    void* ev_;
+    int depth_;
+};
+
+// Joins the object's stream with the caller's for the time of one call.
+class Scope {
+public:
+    explicit Scope(StreamCtx& c) : c_(c) { c_.enter(); }
+    ~Scope() { c_.leave(); }
+    Scope(const Scope&) = delete;
+    Scope& operator=(const Scope&) = delete;
+private:
+    StreamCtx& c_;
+};
+
+// Orders two streams once: everything `later` is given from now on runs after what `earlier` holds now.
+class StreamOrder {
+public:
+    StreamOrder() : turn_(0) { ev_[0] = ev_[1] = nullptr; }
+    StreamOrder(const StreamOrder&) : turn_(0) { ev_[0] = ev_[1] = nullptr; }
+    StreamOrder& operator=(const StreamOrder&) { return *this; }
+    ~StreamOrder() {
+        for (int i = 0; i < 2; ++i)
+            if (ev_[i]) cx_event_destroy(ev_[i]);
+    }
+    void order(void* earlier, void* later) {
+        if (earlier == later) return;
+        void*& ev = ev_[turn_ ^= 1];  // two events in turn: one is never recorded again while its wait is fresh
+        if (!ev) check(cx_event_create(&ev));
+        check(cx_event_record(ev, earlier));
+        check(cx_stream_wait_event(later, ev));
+    }
+private:
+    void* ev_[2];
+    int turn_;
+};
+
+// One handle (scratch, on the object's stream) per object, created on first use so that
+// constructing and cloning threshold/compressor objects never touches the GPU.
 class Handle {
 public:
-    Handle() : h_(nullptr) {}
-    Handle(const Handle&) : h_(nullptr) {}  // clones get their own scratch
+    Handle() : ctx_(std::make_shared<StreamCtx>()), h_(nullptr) {}
+    Handle(const Handle&) : ctx_(std::make_shared<StreamCtx>()), h_(nullptr) {}  // clones get their own scratch and stream
     Handle& operator=(const Handle&) { return *this; }
     ~Handle() { if (h_) cx_destroy(h_); }
     cx_handle get() {
-        if (!h_) check(cx_create(&h_, nullptr));
+        if (!h_) check(cx_create(&h_, ctx_->stream()));
         return h_;
     }
+    StreamCtx& ctx() { return *ctx_; }
+    const std::shared_ptr<StreamCtx>& ctx_ptr() const { return ctx_; }
+    // share another object's stream (a ComprEx and its clones work on one stream)
+    void bind(const std::shared_ptr<StreamCtx>& c) {
+        ctx_ = c;
+        refresh();
+    }
+    // the context's stream changed (StreamCtx::adopt)
+    void refresh() {
+        if (h_) check(cx_set_stream(h_, ctx_->stream()));
+    }
 private:
+    std::shared_ptr<StreamCtx> ctx_;  // outlives the handle: cx_destroy waits for the stream
     cx_handle h_;
 };
 

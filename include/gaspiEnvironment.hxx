@@ -5,8 +5,8 @@
 // A directed channel is identified by (source rank, target rank, tag), as the reference's
 // SourceBuffer::connectToRemoteTarget / TargetBuffer::connectToRemoteSource pair is
 // (src/comprEx.tpp:341-363).  The sender's compressor writes the message straight into the
-// channel's device buffer and the receiver reads it from there: the "transfer" is the
-// stream order of the two kernels.
+// channel's device buffer and the receiver reads it from there: the "transfer" is an event the
+// sender's stream records and the receiver's stream waits for.
 //
 // Two ways to drive the ranks:
 //   * one thread plays all ranks in turn (set_rank before each rank's calls).  A receive with
@@ -36,24 +36,41 @@ struct Channel {
     std::mutex m;
     std::condition_variable cv;
     long long sent = 0, received = 0;  // messages written / consumed
+    // The hand-over on the GPU: the sender records `ready` on its stream behind the kernels that
+    // write the message and the receiver's stream waits for it; the receiver records `freed` behind
+    // the kernels that read it and the next send's stream waits for that (the reference's
+    // notification and the write that waits for it, src/comprEx.tpp:190,231,243).  The counters
+    // above only order the HOST side (who may enqueue what).
+    void* ready = nullptr;
+    void* freed = nullptr;
+    bool ready_set = false, freed_set = false;
 
-    // sender: called after the kernels that write the message were enqueued
-    void post() {
+    ~Channel() {
+        if (ready) cx_event_destroy(ready);
+        if (freed) cx_event_destroy(freed);
+    }
+
+    // sender: called after the kernels that write the message were enqueued on `stream`
+    void post(void* stream) {
         {
             std::lock_guard<std::mutex> g(m);
+            if (!ready) check(cx_event_create(&ready));
+            check(cx_event_record(ready, stream));
+            ready_set = true;
             sent += 1;
         }
         cv.notify_all();
     }
-    // sender, blocking mode: do not overwrite a message nobody has read yet
-    void wait_consumed(bool blocking, double timeout_s) {
-        if (!blocking) return;
+    // sender: do not overwrite a message nobody has read yet.  Blocking mode waits (on the host)
+    // until the receiver has enqueued its reads; either way `stream` then waits for those reads.
+    void wait_consumed(bool blocking, double timeout_s, void* stream) {
         std::unique_lock<std::mutex> g(m);
-        if (!cv.wait_for(g, std::chrono::duration<double>(timeout_s), [&] { return received >= sent; }))
+        if (blocking && !cv.wait_for(g, std::chrono::duration<double>(timeout_s), [&] { return received >= sent; }))
             throw std::runtime_error("Send timed out: the previous message of this channel was never received!");
+        if (freed_set) check(cx_stream_wait_event(stream, freed));
     }
-    // receiver: the reference's TargetBuffer::waitForCompletion
-    void wait_message(bool blocking, double timeout_s) {
+    // receiver: the reference's TargetBuffer::waitForCompletion; `stream` is where the message will be read
+    void wait_message(bool blocking, double timeout_s, void* stream) {
         std::unique_lock<std::mutex> g(m);
         if (!blocking) {
             if (received >= sent)
@@ -61,11 +78,15 @@ struct Channel {
         } else if (!cv.wait_for(g, std::chrono::duration<double>(timeout_s), [&] { return sent > received; })) {
             throw std::runtime_error("Receive timed out: no message arrived!");
         }
+        if (ready_set) check(cx_stream_wait_event(stream, ready));
     }
-    // receiver: called after the kernels that read the message were enqueued
-    void consumed() {
+    // receiver: called after the kernels that read the message were enqueued on `stream`
+    void consumed(void* stream) {
         {
             std::lock_guard<std::mutex> g(m);
+            if (!freed) check(cx_event_create(&freed));
+            check(cx_event_record(freed, stream));
+            freed_set = true;
             received = sent;
         }
         cv.notify_all();
@@ -102,6 +123,15 @@ public:
         timeout_s_ = timeout_s;
     }
     bool blocking() const { return blocking_; }
+    // Not in the reference: the HIP stream on which the calling thread's vectors are produced and
+    // consumed (NULL, the default, = the null stream).  Every exchange call joins its object's own
+    // stream with this one on entry and on exit, so the caller needs no synchronisation of its own.
+    // A per-thread setting, like the rank: each simulated rank may work on a stream of its own.
+    void set_user_stream(void* hip_stream) {
+        tls().stream_env = this;
+        tls().user_stream = hip_stream;
+    }
+    void* user_stream() { return tls().stream_env == this ? tls().user_stream : nullptr; }
     double timeout_s() const { return timeout_s_; }
 
     // all ranks' threads meet here (blocking mode); a no-op when one thread plays every rank
@@ -145,6 +175,8 @@ private:
     struct Tls {
         GaspiEnvironment* env = nullptr;
         int rank = 0;
+        GaspiEnvironment* stream_env = nullptr;
+        void* user_stream = nullptr;
     };
     static Tls& tls() {
         static thread_local Tls t;

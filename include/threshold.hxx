@@ -15,6 +15,7 @@
 #define THRESHOLD_H
 
 #include <cmath>
+#include <memory>
 #include <stdexcept>
 
 #include "cx_device.hxx"
@@ -28,6 +29,7 @@ public:
     virtual void apply(VarTYPE* out_vec, int out_vec_size, const VarTYPE* in_vec, int in_vec_size) {
         if (out_vec_size < in_vec_size)
             throw std::runtime_error("Thresholding target buffer is smaller than source buffer!");
+        cxx::Scope scope(handle_.ctx());
         prepare(in_vec, in_vec_size);
         run_apply(out_vec, nullptr, in_vec, in_vec_size);
     }
@@ -37,6 +39,7 @@ public:
                              const VarTYPE* in_vec, int in_vec_size) {
         if (high_vec_size < in_vec_size || low_vec_size < in_vec_size)
             throw std::runtime_error("Thresholding target buffer is smaller than source buffer!");
+        cxx::Scope scope(handle_.ctx());
         prepare(in_vec, in_vec_size);
         run_apply(high_vec, low_vec, in_vec, in_vec_size);
     }
@@ -53,6 +56,11 @@ public:
     virtual const VarTYPE* device_threshold() { return nullptr; }
     // Not in the reference: sizes the GPU scratch of this threshold for vectors of up to n elements.
     virtual void reserve(int n) {}
+    // Not in the reference: the stream this object's GPU work runs on and the caller's stream it is
+    // joined with around every call (cx_device.hxx).  A ComprEx binds its clones to its own.
+    void bind_stream(const std::shared_ptr<cxx::StreamCtx>& ctx) { handle_.bind(ctx); }
+    cxx::StreamCtx& stream_context() { return handle_.ctx(); }
+    void stream_changed() { handle_.refresh(); }
 
     // Not in the reference.  True when prepare_with on n elements would apply the top-k rule to
     // every element (no sub-sampling); the fraction is returned.  ComprEx then computes threshold
@@ -146,6 +154,7 @@ public:
         sample_m_ = 0;
         if (m <= 0) return;
         if (!idx) throw std::runtime_error("sample positions: null pointer");
+        cxx::Scope scope(this->handle_.ctx());
         cx_handle h = this->handle_.get();
         cxx::check(cx_copy(h, sample_idx_.reserve((size_t)m * sizeof(int)), idx, (size_t)m * sizeof(int)));
         cxx::check(cx_synchronize(h));
@@ -193,6 +202,7 @@ public:
             prepare_indexed(vec, vec_size, nullptr, static_cast<const int*>(sample_idx_.data()), sample_m_);
             return;
         }
+        cxx::Scope scope(this->handle_.ctx());
         cx_handle h = this->handle_.get();
         cxx::Staged<const VarTYPE> v(h, this->stage_in_, vec, (size_t)vec_size, true, false);
         cxx::check(cx_topk_threshold(h, cxx::dtype_of<VarTYPE>::value, v.get(), nullptr, vec_size, 0, topK,
@@ -207,6 +217,7 @@ public:
             prepare_indexed(vec, vec_size, add_vec, static_cast<const int*>(sample_idx_.data()), sample_m_);
             return;
         }
+        cxx::Scope scope(this->handle_.ctx());
         cx_handle h = this->handle_.get();
         cxx::Staged<const VarTYPE> v(h, this->stage_in_, vec, (size_t)vec_size, true, false);
         cxx::Staged<const VarTYPE> a(h, this->stage_hi_, add_vec, (size_t)add_vec_size, true, false);
@@ -219,6 +230,7 @@ public:
     // Not in the reference: the same order statistic over caller-chosen sample positions
     // (device int32 indices).
     void prepare_indexed(const VarTYPE* vec, int vec_size, const VarTYPE* add_vec, const int* d_idx, int m) {
+        cxx::Scope scope(this->handle_.ctx());
         cx_handle h = this->handle_.get();
         cxx::Staged<const VarTYPE> v(h, this->stage_in_, vec, (size_t)vec_size, true, false);
         cxx::Staged<const VarTYPE> a(h, this->stage_hi_, add_vec, (size_t)(add_vec ? vec_size : 0), true, false);

@@ -23,7 +23,7 @@ template <typename T> struct PeekComprEx : ComprEx<T> {
         cxx::check(cx_synchronize(this->handle_.get()));
         return out;
     }
-    void drop() { this->targBuff_data->consumed(); }
+    void drop() { this->targBuff_data->consumed(this->stream()); }
 };
 
 struct Lcg {

@@ -16,7 +16,7 @@ BIN = os.path.join(ROOT, "tests", "cpp", "bin")
 
 
 @pytest.mark.parametrize("name", ["threshold_test", "compressor_test", "comprex_test", "fast_comprex_test", "allreduce_test",
-                                  "tf_ops_test", "capi_test"])
+                                  "tf_ops_test", "capi_test", "streams_test"])
 def test_cpp_mirror_of_reference_tests(name):
     exe = os.path.join(BIN, name)
     assert os.path.exists(exe), "build tests/cpp first (make -C tests/cpp, or __graft_entry__.build())"
