@@ -64,6 +64,9 @@ void GaspiEnvironment_set_rank(void* self, int rank, int ranks) {
 void GaspiEnvironment_set_blocking(void* self, int blocking, double timeout_s) {
     static_cast<GaspiEnvironment*>(self)->set_blocking(blocking != 0, timeout_s);
 }
+void GaspiEnvironment_set_user_stream(void* self, void* hip_stream) {
+    static_cast<GaspiEnvironment*>(self)->set_user_stream(hip_stream);
+}
 void Gaspi_Printf(const char* msg) {
     printf("%s\n", msg);
     fflush(stdout);

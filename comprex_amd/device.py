@@ -177,13 +177,16 @@ class Handle:
                                         C.byref(nbytes) if sync else None))
         return nbytes.value if sync else None
 
-    def add(self, out, msg, check_header=True):
-        check(self.lib.cx_ip_add(self._h, _dt(out), _p(out), out.numel(), _p(msg), 1 if check_header else 0))
+    def add(self, out, msg, check_header=True, any_order=False):
+        """any_order: look at the indices first (one more wait) and apply a message that is not
+        index-sorted pair after pair, as the reference's loop does (CX_ADD_ANY_ORDER)."""
+        check(self.lib.cx_ip_add(self._h, _dt(out), _p(out), out.numel(), _p(msg),
+                                 2 if any_order else (1 if check_header else 0)))
 
-    def reduce(self, out, msgs, accumulate=False, mode=0):
+    def reduce(self, out, msgs, accumulate=False, mode=0, any_order=False):
         arr = (C.c_void_p * len(msgs))(*[m.data_ptr() for m in msgs])
         check(self.lib.cx_ip_reduce(self._h, _dt(out), _p(out), out.numel(), arr, len(msgs),
-                                    1 if accumulate else 0, int(mode)))
+                                    1 if accumulate else 0, int(mode) | (4 if any_order else 0)))
 
     # ---- residual maintenance ---------------------------------------------
     def zero(self, v):

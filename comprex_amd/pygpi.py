@@ -33,6 +33,7 @@ _PROTOS = {
     "ThresholdTopK_new": (_vp, [_f]), "ThresholdTopK_del": (None, [_vp]),
     "ThresholdTopK_getThreshold": (_f, [_vp]),
     "GaspiEnvironment_set_blocking": (None, [_vp, _i, C.c_double]),
+    "GaspiEnvironment_set_user_stream": (None, [_vp, _vp]),
     "CompressorNone_new": (_vp, []), "CompressorNone_del": (None, [_vp]),
     "CompressorRLE_new": (_vp, []), "CompressorRLE_del": (None, [_vp]),
     "CompressorIndexPairs_new": (_vp, []), "CompressorIndexPairs_del": (None, [_vp]),
@@ -112,6 +113,13 @@ class GaspiEnvironment(Getable):
     def set_blocking(self, blocking, timeout_s=60.0):
         """Not in the reference: one host thread per rank; receives wait for their message."""
         libcomprex().GaspiEnvironment_set_blocking(self.obj, int(blocking), float(timeout_s))
+
+    def set_user_stream(self, stream):
+        """Not in the reference: the stream the calling thread's device vectors live on (a
+        torch.cuda.Stream, a raw hipStream_t as an int, or None for the null stream).  Every exchange
+        call joins its object's own stream with it on entry and on exit."""
+        raw = getattr(stream, "cuda_stream", stream)
+        libcomprex().GaspiEnvironment_set_user_stream(self.obj, C.c_void_p(raw or None))
 
     def barrier(self):
         libcomprex().GaspiEnvironment_barrier(self.obj)

@@ -318,6 +318,10 @@ void CompressorIndexPairs_del(void* self);
  * from that rank's own host thread (GaspiEnvironment_set_rank, then GaspiEnvironment_set_blocking so
  * that receives wait for their message); apply/flush work in place on `data`, host or device. */
 void GaspiEnvironment_set_blocking(void* self, int blocking, double timeout_s);
+/* No counterpart in the reference (its vectors are host memory).  The HIP stream on which the
+ * calling thread's device vectors are produced and consumed (NULL, the default, = the null stream):
+ * every exchange call joins its object's own stream with it on entry and on exit. */
+void GaspiEnvironment_set_user_stream(void* self, void* hip_stream);
 void* Comprex_AllToOneAllreduce_new(void* gaspi_env);
 void Comprex_AllToOneAllreduce_del(void* self);
 void Comprex_AllToOneAllreduce_setupConnections(void* self, int size, int tag, int chiefRank, float compression_ratio,

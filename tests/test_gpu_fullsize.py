@@ -189,6 +189,19 @@ def test_c5_sparse_reduce_eight_ranks(dev, oracle):
     want = rests.cpu().numpy() + got
     dev.add_vec(rests, torch.from_numpy(got).cuda())
     assert rests.cpu().numpy().tobytes() == want.tobytes()
+    # ... and the chief's broadcast leg as the reference runs it (src/allreduce.tpp:205): writeRemote
+    # of the reduced vector into a residual, exact top-k 1 %, against the checker
+    topk, ds = np.float32(0.01), 1 << 27
+    rests_h = np.random.default_rng(10).standard_normal(n).astype(np.float32)
+    rests = torch.from_numpy(rests_h.copy()).cuda()
+    want_msg, want_thr = oracle.write_remote(rests_h, got, topk, ds)
+    dense = torch.from_numpy(got).cuda()
+    buf = torch.zeros(8 + 8 * (n // 50), dtype=torch.uint8, device="cuda")
+    thr = dev.topk_threshold(rests, dense, topk, ds)
+    nbytes = dev.compress(buf, dense, rests)
+    assert thr == want_thr and nbytes == want_msg.size
+    assert buf[:nbytes].cpu().numpy().tobytes() == want_msg.tobytes()
+    assert rests.cpu().numpy().tobytes() == rests_h.tobytes()
     dev.synchronize()
 
 

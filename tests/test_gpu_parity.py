@@ -701,6 +701,74 @@ def test_tiled_reduce_reports_unsorted_message(dev):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_add_and_reduce_take_any_index_order_when_asked(dev, oracle, dtype):
+    """The reference's add walks the pairs as stored (src/compressor.hxx:640-658): any index order, an
+    index repeated anywhere, the additions in message order.  The fast paths want ascending indices.
+    With CX_ADD_ANY_ORDER / CX_REDUCE_ANY_ORDER (what Compressor::add / add_many pass) the call looks
+    at the indices first and applies such messages pair after pair: expected values from the
+    checker, which is that loop.  Without the flag the disorder is reported (CX_ERR_INDEX), never
+    turned into a different sum silently."""
+    from comprex_amd.device import ComprexError
+    from comprex_amd import _lib
+    rng = np.random.default_rng(43)
+    n, k = 40_000, 7_003
+    rec = np.dtype([("i", np.int32), ("v", dtype)])
+
+    def message(sorted_idx):
+        idx = rng.integers(0, n // 8, k).astype(np.int32)            # many repeats, far apart
+        idx[200:210] = idx[3000]                                       # and a run of repeats inside one chunk
+        if sorted_idx:
+            idx = np.sort(idx)
+        body = np.empty(k, rec)
+        body["i"], body["v"] = idx, _rand(rng, k, dtype)
+        return np.concatenate([np.array([n, k], np.int32).view(np.uint8), body.view(np.uint8)])
+
+    msgs = [message(False), message(True), message(False), message(False), message(True)]
+    start = _rand(rng, n, dtype)
+    # one message at a time
+    want = start.copy()
+    g = torch.from_numpy(start.copy()).cuda()
+    for m in msgs:
+        oracle.ip_add(m, want)
+        dev.add(g, _gpu(m), any_order=True)
+    dev.synchronize()
+    assert g.cpu().numpy().tobytes() == want.tobytes()
+    # all at once, added into the vector and from zeros
+    gm = [_gpu(m) for m in msgs]
+    g = torch.from_numpy(start.copy()).cuda()
+    dev.reduce(g, gm, accumulate=True, any_order=True)
+    dev.synchronize()
+    assert g.cpu().numpy().tobytes() == want.tobytes()
+    want0 = np.zeros(n, dtype)
+    for m in msgs:
+        oracle.ip_add(m, want0)
+    g = torch.full((n,), 5, dtype=NP2T[dtype], device="cuda")
+    dev.reduce(g, gm, accumulate=False, any_order=True)
+    dev.synchronize()
+    assert g.cpu().numpy().tobytes() == want0.tobytes()
+    # sorted messages keep the fast path and its result
+    sorted_only = [gm[1], gm[4]]
+    wants = start.copy()
+    oracle.ip_add(msgs[1], wants)
+    oracle.ip_add(msgs[4], wants)
+    g = torch.from_numpy(start.copy()).cuda()
+    dev.reduce(g, sorted_only, accumulate=True, any_order=True)
+    dev.synchronize()
+    assert g.cpu().numpy().tobytes() == wants.tobytes()
+    # without the flag: reported
+    g = torch.zeros(n, dtype=NP2T[dtype], device="cuda")
+    dev.add(g, gm[0], check_header=False)
+    with pytest.raises(ComprexError) as e:
+        dev.synchronize()
+    assert e.value.code == _lib.CX_ERR_INDEX
+    for acc in (False, True):
+        dev.reduce(g, gm, accumulate=acc)
+        with pytest.raises(ComprexError) as e:
+            dev.synchronize()
+        assert e.value.code == _lib.CX_ERR_INDEX
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_decompress_takes_any_index_order_when_it_reports_back(dev, oracle, dtype):
     """The reference's decoder walks the pairs as stored (src/compressor.hxx:613-633): any index order,
     an index repeated anywhere, the last value wins.  The fast path wants ascending indices; a

@@ -1,7 +1,8 @@
 """cx_ip_compress_noalloc (scratch in a static device array) against cx_ip_compress (scratch the
-handle allocates), through the C ABI: same message bytes, size prefix and residual, bit for bit, on
-two calls in a row, the second with a smaller input, so that the static array still holds the first
-call's contents when the second one runs."""
+handle allocates) AND against the CPU checker, through the C ABI: same message bytes, size prefix
+and residual, bit for bit, on calls in a row, the later ones with smaller inputs, so that the static
+array still holds an earlier call's contents when they run; for every tile shape, for sub-vectors at
+odd offsets (the scalar path) and at the largest size the entry point takes."""
 import ctypes as C
 
 import numpy as np
@@ -49,14 +50,27 @@ def _run(L, h, entry, dtype, data, update, thr, cap_bytes):
     return msg[:nbytes].cpu().numpy().tobytes(), nbytes, None if update is None else update.cpu().numpy().tobytes()
 
 
+def _checker(oracle, data, update, thr):
+    """The same compress through the CPU checker: (message bytes, byte count, residual bytes)."""
+    d = None if data is None else data.cpu().numpy()
+    u = None if update is None else update.cpu().numpy().copy()
+    msg = oracle.ip_compress(d, u, thr)
+    return msg.tobytes(), msg.size, None if u is None else u.tobytes()
+
+
+@pytest.mark.parametrize("offset", [0, 1])
+@pytest.mark.parametrize("items", [2, 4, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.int32])
-def test_noalloc_matches_allocating_entry_point_on_consecutive_calls(dtype):
+def test_noalloc_matches_allocating_entry_point_and_checker_on_consecutive_calls(oracle, dtype, items, offset):
+    """offset 1: the vectors start one element behind an aligned address (scalar loads, the tile
+    shape of that path); items: 16-byte loads per lane and tile of the vector path."""
     L = _lib.lib()
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream()
     h = C.c_void_p()
     _lib.check(L.cx_create(C.byref(h), C.c_void_p(stream.cuda_stream)))
     try:
+        _lib.check(L.cx_set_option(h, b"compact_items", items))
         rng = np.random.default_rng(5)
         esize = torch.empty((), dtype=dtype).element_size()
         # a large call, then a smaller one (odd length: ragged last tile), then a dense flush-like call
@@ -64,19 +78,49 @@ def test_noalloc_matches_allocating_entry_point_on_consecutive_calls(dtype):
         for n, thr, mode in cases:
             if dtype == torch.int32:
                 thr = int(thr * 400)
-            g, r = _inputs(rng, n, dtype)
+            g, r = _inputs(rng, n + offset, dtype)
+            g, r = g[offset:], r[offset:]
             cap = 8 + n * (4 + esize)
             want_in = (g if mode != "update" else None, r.clone() if mode != "data" else None)
             got_in = (g if mode != "update" else None, r.clone() if mode != "data" else None)
+            if offset:  # clone() realigns: keep the odd start
+                hold_w, hold_g = torch.empty(n + 1, dtype=dtype, device="cuda"), torch.empty(n + 1, dtype=dtype, device="cuda")
+                if want_in[1] is not None:
+                    hold_w[1:].copy_(r), hold_g[1:].copy_(r)
+                    want_in, got_in = (want_in[0], hold_w[1:]), (got_in[0], hold_g[1:])
+            check_in = (want_in[0], None if want_in[1] is None else want_in[1].clone())
             want = _run(L, h, "cx_ip_compress", dtype, want_in[0], want_in[1], thr, cap)
             torch.cuda.synchronize()
             free_before = torch.cuda.mem_get_info()[0]
             got = _run(L, h, "cx_ip_compress_noalloc", dtype, got_in[0], got_in[1], thr, cap)
             assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
-            assert got[1] == want[1], (n, mode, got[1], want[1])
-            assert got[0] == want[0], "message differs (n=%d, %s)" % (n, mode)
-            assert got[2] == want[2], "residual differs (n=%d, %s)" % (n, mode)
+            ref = _checker(oracle, check_in[0], check_in[1], thr)
+            assert got[1] == want[1] == ref[1], (n, mode, got[1], want[1], ref[1])
+            assert got[0] == want[0], "message differs from the allocating entry point (n=%d, %s)" % (n, mode)
+            assert got[0] == ref[0], "message differs from the checker (n=%d, %s)" % (n, mode)
+            assert got[2] == want[2] == ref[2], "residual differs (n=%d, %s)" % (n, mode)
             assert want[1] > 8 or thr > 100, "the case selects nothing"
+    finally:
+        L.cx_destroy(h)
+
+
+def test_noalloc_largest_fp64_vector_smallest_tiles(oracle):
+    """fp64 at exactly cx_noalloc_max_elements() with the smallest tile shape: the case that needs the
+    most of the static array (staging slots of 3 words per pair, the most tiles)."""
+    L = _lib.lib()
+    torch.cuda.set_device(0)
+    h = C.c_void_p()
+    _lib.check(L.cx_create(C.byref(h), C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    try:
+        _lib.check(L.cx_set_option(h, b"compact_items", 2))
+        n = int(L.cx_noalloc_max_elements())
+        rng = np.random.default_rng(6)
+        g = torch.from_numpy(rng.standard_normal(n)).cuda()
+        r = torch.from_numpy(0.3 * rng.standard_normal(n)).cuda()
+        cap = 8 + 12 * (n // 20)
+        ref = _checker(oracle, g, r, 2.4)
+        got = _run(L, h, "cx_ip_compress_noalloc", torch.float64, g, r, 2.4, cap)
+        assert 8 < got[1] == ref[1] and got[0] == ref[0] and got[2] == ref[2]
     finally:
         L.cx_destroy(h)
 
