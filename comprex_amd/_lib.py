@@ -71,6 +71,7 @@ def lib():
         "cx_noalloc_max_elements": (ll, []),
         "cx_reserve": (i, [vp, i, i, C.c_uint]),
         "cx_ip_compress_topk": (i, [vp, i, vp, ll, vp, vp, i, C.c_float, vp, vp, C.POINTER(i)]),
+        "cx_ip_write_step": (i, [vp, i, vp, ll, vp, vp, i, C.c_float, i, C.c_float, vp, i, vp, vp, C.POINTER(i)]),
         "cx_get_option": (i, [vp, C.c_char_p, C.POINTER(i)]),
         "cx_rle_compress": (i, [vp, i, vp, ll, vp, vp, i, vp, vp, vp, C.POINTER(i)]),
         "cx_rle_decompress": (i, [vp, i, vp, i, vp, C.POINTER(i)]),

@@ -126,6 +126,45 @@ int compress_topk_impl(cx_handle h, void* out_msg, long long out_capacity, const
     return rc;
 }
 
+// ThresholdTopK::prepare_with + compress_add_update in one call
+template <typename T>
+int write_step_impl(cx_handle h, void* out_msg, long long out_capacity, const void* data, void* update, int n, float topK,
+                    int default_subsamples, float subsample_factor, const int* d_idx, int m, void* d_thr_out,
+                    int* d_size_prefix, int* h_bytes) {
+    const T* d = static_cast<const T*>(data);
+    T* u = static_cast<T*>(update);
+    T* thr = static_cast<T*>(d_thr_out);
+    int mode, keys;
+    float stepsize = 1.0f;
+    if (d_idx && m > 0) {
+        mode = kSampleIndexed;
+        keys = m;
+    } else {
+        int subsamples = cx_topk_subsamples(topK, default_subsamples, subsample_factor);
+        if (subsamples < 0) subsamples = 0x7fffffff;  // undefined in the reference: use the whole vector
+        if (n < subsamples) {
+            mode = kSampleFull;
+            keys = n;
+        } else {
+            mode = kSampleStrided;
+            keys = subsamples;
+            stepsize = (float)n / (float)subsamples;
+        }
+    }
+    int rc;
+    if (mode == kSampleFull) {
+        rc = launch_compress_topk<T>(h, out_msg, out_capacity, d, u, n, topK, thr, d_size_prefix);
+    } else {
+        rc = launch_topk_threshold<T>(h, u, d, n, d_idx, keys, mode, stepsize, topK, thr);
+        if (rc == CX_OK) rc = launch_compact<T>(h, out_msg, out_capacity, d, u, n, nullptr, thr, d_size_prefix);
+    }
+    if (rc != CX_OK || !h_bytes) return rc;
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 8, out_msg, 8, hipMemcpyDeviceToHost, h->stream));
+    rc = collect_status(h);
+    *h_bytes = 8 + h->h_pinned[9] * 4 * Elem<T>::pair_words;
+    return rc;
+}
+
 template <typename T>
 int rle_compress_impl(cx_handle h, void* out_msg, long long out_capacity, const void* data, void* update, int n,
                       const void* thr_host, const void* d_thr, int* d_size_prefix, int* h_bytes) {
@@ -378,6 +417,7 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         h->fused_topk = value ? 1 : 0;
     } else if (!strcmp(key, "select_short_list")) {
         h->select_short_list = value ? 1 : 0;
+
     } else {
         return fail(CX_ERR_INVALID, "unknown option '%s'", key);
     }
@@ -497,6 +537,16 @@ int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_c
     if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
     CX_DISPATCH(dt, compress_topk_impl<T>(h, out_msg, out_capacity, data, update, n, topK, d_thr_out, d_size_prefix,
                                           h_bytes));
+}
+
+int cx_ip_write_step(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,
+                     int n, float topK, int default_subsamples, float subsample_factor, const int* d_idx, int m,
+                     void* d_thr_out, int* d_size_prefix, int* h_bytes) {
+    if (!h) return fail(CX_ERR_INVALID, "null handle");
+    if (n < 0 || !update || !data || m < 0) return fail(CX_ERR_INVALID, "write_step: needs both vectors and sizes >= 0");
+    if (topK > 1.0f || topK < 0.0f) return fail(CX_ERR_TOPK, "topK value must be between 0.0 and 1.0!");
+    CX_DISPATCH(dt, write_step_impl<T>(h, out_msg, out_capacity, data, update, n, topK, default_subsamples,
+                                       subsample_factor, d_idx, m, d_thr_out, d_size_prefix, h_bytes));
 }
 
 int cx_rle_compress(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity, const void* data, void* update,

@@ -58,10 +58,7 @@ constexpr int kMaxRadixPasses = 6; // 63-bit keys, 11 bits per pass
 
 // State of one radix-select run; lives in device memory.
 struct SelectState {
-    unsigned long long prefix;     // key bits fixed so far
-    unsigned long long mask;       // which bits of `prefix` are fixed
-    unsigned long long rank;       // descending rank still to find among matching keys
-    unsigned int hist[kRadixBins]; // digit histogram of the current pass
+    unsigned int hist[kRadixBins]; // two-launch select: top-digit counts of all keys; zero between runs
     unsigned int short_count;      // two-launch select: keys in the short list; zero between runs
     unsigned int short_digit;      // ... and the largest cut of a block: the leading two digits of its short_k-th key
     // chained passes (no pick launch in between): one histogram per pass, all zero between runs,
@@ -137,6 +134,9 @@ struct cx_handle_s {
 
 namespace cx {
 
+// sample_mode of launch_topk_threshold
+enum { kSampleFull = 0, kSampleStrided = 1, kSampleIndexed = 2 };
+
 // ---- launchers implemented in the k_*.hip files -----------------------------
 template <typename T>
 int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
@@ -184,8 +184,5 @@ template <typename T> int launch_zero(cx_handle h, T* v, int n);
 template <typename T> int launch_add_vec(cx_handle h, T* data, const T* rests, int n);
 template <typename T>
 int launch_threshold_apply(cx_handle h, T* high, T* low, const T* in, int n, const T* thr_host, const T* d_thr);
-
-// sample_mode of launch_topk_threshold
-enum { kSampleFull = 0, kSampleStrided = 1, kSampleIndexed = 2 };
 
 }  // namespace cx

@@ -40,15 +40,6 @@ __device__ __forceinline__ void hist_add(unsigned* lds_hist, bool active, unsign
     if (active && digit != d0) atomicAdd(&lds_hist[digit], 1u);
 }
 
-__global__ __launch_bounds__(kBlock) void select_init_kernel(SelectState* st, unsigned long long rank) {
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) st->hist[b] = 0u;
-    if (threadIdx.x == 0) {
-        st->prefix = 0ull;
-        st->mask = 0ull;
-        st->rank = rank;
-    }
-}
-
 // Adds a block's LDS digit counts to the global histogram.
 template <int BLOCK> __device__ __forceinline__ void merge_hist(const unsigned* lds_hist, SelectState* st) {
     __syncthreads();
@@ -58,38 +49,26 @@ template <int BLOCK> __device__ __forceinline__ void merge_hist(const unsigned* 
     }
 }
 
-// Picks the digit that holds the wanted descending rank, narrows the state, clears the
-// histogram for the next pass.  After the last pass the key is complete and the
-// threshold is written.  One block.  (Folding this into the histogram kernel, with the block
-// that arrives last doing the pick, was measured slower on this GPU: the device-scope fences
-// that make the other blocks' counts visible inside one kernel cost more than a launch.)
+// Last step of the chained passes: the pick over the last pass's histogram completes the key; the
+// threshold is written and the passes' histograms are cleared for the next run.  One block.
+// (Folding a pick into the histogram kernel, with the block that arrives last doing it, was measured
+// slower on this GPU: the device-scope fences that make the other blocks' counts visible inside one
+// kernel cost more than a launch.  Chaining does without: see state_entering_pass.)
 template <typename T>
-__global__ __launch_bounds__(kBlock) void select_pick_kernel(SelectState* st, int shift, int bits, int last,
-                                                             int plus_one, T* __restrict__ thr_out) {
+__global__ __launch_bounds__(kBlock) void select_final_kernel(SelectState* st, unsigned long long rank0, int plus_one,
+                                                              T* __restrict__ thr_out) {
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
+    using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
     __shared__ unsigned long long s_above, s_sum[kBlock / 64];
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
-        lds_hist[b] = st->hist[b];
-        st->hist[b] = 0u;
-    }
-    __syncthreads();
-    const unsigned long long rank = st->rank;
-    unsigned digit;
-    unsigned long long above;
-    block_pick<kBlock>(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+    const PickState done = state_entering_pass<T, kBlock>(st, kPasses, rank0, lds_hist, s_sum, &s_digit, &s_above);
     if (threadIdx.x == 0) {
-        const unsigned long long prefix = st->prefix | ((unsigned long long)digit << shift);
-        st->prefix = prefix;
-        st->mask = st->mask | (((1ull << bits) - 1ull) << shift);
-        st->rank = rank - above;
-        if (last) {
-            using key_t = typename Elem<T>::key_t;
-            T v = value_of((key_t)prefix, T());
-            if (plus_one) v = (T)(v + 1);
-            *thr_out = v;
-        }
+        T v = value_of((key_t)done.prefix, T());
+        if (plus_one) v = (T)(v + 1);
+        *thr_out = v;
     }
+    for (int b = threadIdx.x; b < kPasses * kRadixBins; b += kBlock) (&st->pass_hist[0][0])[b] = 0u;
 }
 
 // One histogram pass over the keys described by (vec, add, idx).  SMODE: 0 whole vector,
@@ -97,15 +76,28 @@ __global__ __launch_bounds__(kBlock) void select_pick_kernel(SelectState* st, in
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
 __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                              const int* __restrict__ idx, long long m, int n,
-                                                             float stepsize, SelectState* __restrict__ st, int shift,
-                                                             int bits) {
+                                                             float stepsize, SelectState* __restrict__ st, int p,
+                                                             unsigned long long rank0) {
     using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit;
+    __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    // chained passes: every block redoes the cheap pick over the previous pass's complete histogram
+    PickState s;
+    s.prefix = 0ull;
+    s.mask = 0ull;
+    s.rank = rank0;
+    if (p > 0) {
+        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above);
+        if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
+    }
     for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
     __syncthreads();
 
-    const key_t prefix = (key_t)st->prefix;
-    const key_t mask = (key_t)st->mask;
+    const key_t prefix = (key_t)s.prefix;
+    const key_t mask = (key_t)s.mask;
+    int shift, bits;
+    pass_digits_dev<T>(p, shift, bits);
     const unsigned digit_mask = (1u << bits) - 1u;
     const long long stride = (long long)gridDim.x * kBlock;
 
@@ -153,7 +145,11 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
             if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
         }
     }
-    merge_hist<kBlock>(lds_hist, st);
+    __syncthreads();
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+        const unsigned c = lds_hist[b];
+        if (c) atomicAdd(&st->pass_hist[p][b], c);
+    }
 }
 
 // One histogram pass over the values of an IndexPairs message (int32 n | int32 k | k pairs), whose
@@ -711,41 +707,28 @@ __global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restr
 template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v; }
 
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
-void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long long m, int n, float stepsize, int shift,
-                 int bits) {
+void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long long m, int n, float stepsize, int p,
+                 unsigned long long rank0) {
     const long long per_block = (long long)kBlock * VEC * 8;
     long long blocks = (m + per_block - 1) / per_block;
     if (blocks < 1) blocks = 1;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL((select_hist_kernel<T, SMODE, HAS_ADD, VEC>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
-                       vec, add, idx, m, n, stepsize, h->sel, shift, bits);
+                       vec, add, idx, m, n, stepsize, h->sel, p, rank0);
 }
 
 template <typename T, bool HAS_ADD>
 void dispatch_hist(cx_handle h, int smode, bool vec_ok, const T* vec, const T* add, const int* idx, long long m, int n,
-                   float stepsize, int shift, int bits) {
+                   float stepsize, int p, unsigned long long rank0) {
     constexpr int kVec = 16 / (int)sizeof(T);
     if (smode == kSampleFull) {
-        if (vec_ok) launch_hist<T, 0, HAS_ADD, kVec>(h, vec, add, idx, m, n, stepsize, shift, bits);
-        else launch_hist<T, 0, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, shift, bits);
+        if (vec_ok) launch_hist<T, 0, HAS_ADD, kVec>(h, vec, add, idx, m, n, stepsize, p, rank0);
+        else launch_hist<T, 0, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
     } else if (smode == kSampleStrided) {
-        launch_hist<T, 1, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, shift, bits);
+        launch_hist<T, 1, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
     } else {
-        launch_hist<T, 2, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, shift, bits);
+        launch_hist<T, 2, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
     }
-}
-
-// Shift and width of radix pass p of a key of Elem<T>::key_bits bits.
-template <typename T> void pass_digits(int p, int* shift, int* bits, int* last) {
-    constexpr int kKeyBits = Elem<T>::key_bits;
-    constexpr int kPasses = (kKeyBits + kRadixBits - 1) / kRadixBits;
-    *shift = kKeyBits - kRadixBits * (p + 1);
-    *bits = kRadixBits;
-    if (*shift < 0) {
-        *bits += *shift;
-        *shift = 0;
-    }
-    *last = p == kPasses - 1 ? 1 : 0;
 }
 
 }  // namespace
@@ -825,17 +808,14 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
 
     const bool vec_ok =
         ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
-    hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank);
+    // chained radix passes (no pick launch in between), then the last pick
     for (int p = 0; p < kPasses; ++p) {
-        int shift, bits, last;
-        pass_digits<T>(p, &shift, &bits, &last);
         if (add_vec)
-            dispatch_hist<T, true>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, shift, bits);
+            dispatch_hist<T, true>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank);
         else
-            dispatch_hist<T, false>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, shift, bits);
-        hipLaunchKernelGGL(select_pick_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, shift, bits, last,
-                           plus_one, d_thr_out);
+            dispatch_hist<T, false>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank);
     }
+    hipLaunchKernelGGL(select_final_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank, plus_one, d_thr_out);
     CX_HIP(hipGetLastError());
     return CX_OK;
 }

@@ -138,6 +138,20 @@ class Handle:
             update.numel(), float(topk), _p(d_thr), _p(size_prefix), C.byref(nbytes)))
         return nbytes.value
 
+    def write_step(self, out_msg, data, update, topk, default_subsamples=1000, subsample_factor=10.0, idx=None,
+                   d_thr=None, size_prefix=None, sync=True):
+        """ThresholdTopK(topk, default_subsamples, subsample_factor).prepare_with(update, data) and
+        compress_add_update in one call (cx_ip_write_step); idx: int32 device tensor of sample
+        positions instead of the strided rule.  Returns bytes written when sync."""
+        if data.numel() != update.numel():
+            raise ComprexError(_lib.CX_ERR_SIZE_MISMATCH, "vector sizes must be the same!")
+        nbytes = C.c_int(0)
+        check(self.lib.cx_ip_write_step(
+            self._h, _dt(update), _p(out_msg), out_msg.numel() * out_msg.element_size(), _p(data), _p(update),
+            update.numel(), float(topk), int(default_subsamples), float(subsample_factor), _p(idx),
+            0 if idx is None else idx.numel(), _p(d_thr), _p(size_prefix), C.byref(nbytes) if sync else None))
+        return nbytes.value if sync else None
+
     def get_option(self, key):
         v = C.c_int(0)
         check(self.lib.cx_get_option(self._h, key.encode(), C.byref(v)))

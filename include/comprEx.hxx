@@ -114,16 +114,16 @@ protected:
     }
 
     // residual += d_data with the entries above the threshold compressed into the message at
-    // `d_target`: one fused call when the threshold is a whole-vector top-k and the compressor
-    // has a path for it, else false (nothing done) and the caller takes the two steps.
+    // `d_target`: one call when the threshold is a top-k rule and the compressor has a path for
+    // it, else false (nothing done) and the caller takes the two steps.
     bool fused_topk_into(void* d_target, long long capacity, const VarTYPE* d_data, int n, int* d_size_prefix) {
-        float topK = 0;
-        if (n != rests_size || n <= 0 || !threshold->whole_vector_topk(n, &topK)) return false;
-        if (topK > 1.0f || topK < 0.0f) return false;  // let prepare_with report it
+        typename ThresholdFunction<VarTYPE>::TopKRule rule;
+        if (n != rests_size || n <= 0 || !threshold->topk_rule(&rule)) return false;
+        if (rule.topK > 1.0f || rule.topK < 0.0f) return false;  // let prepare_with report it
         // a claim without a fused call is harmless: the caller's prepare_with follows and overwrites it
         VarTYPE* slot = threshold->claim_device_threshold();
         if (!slot) return false;
-        return compressor->compress_topk_device(d_target, capacity, d_data, rests(), n, topK, slot, d_size_prefix);
+        return compressor->write_step_device(d_target, capacity, d_data, rests(), n, rule, slot, d_size_prefix);
     }
 
 public:
@@ -278,8 +278,8 @@ public:
         cxx::Scope scope(joined());
         cx_handle h = handle_.get();
         cxx::Staged<const VarTYPE> v(h, stage_, vector, (size_t)size, true, false);
-        float topK = 0;
-        if (size == rests_size && threshold->whole_vector_topk(size, &topK)) {
+        typename ThresholdFunction<VarTYPE>::TopKRule rule;
+        if (size == rests_size && size > 0 && threshold->topk_rule(&rule)) {
             wait_for_room();
             const int offset = send_sizeBytes ? (int)sizeof(int) : 0;
             if (fused_topk_into(src_address() + offset, bufferSize - offset, v.get(), size,

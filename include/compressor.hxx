@@ -99,11 +99,12 @@ public:
     virtual int decompress_device(VarTYPE* d_output, int output_size, const void* d_source, bool wait) = 0;
     virtual void add_device(VarTYPE* d_output, int output_size, const void* d_source) = 0;
 
-    // Not in the reference.  Whole-vector ThresholdTopK(topK)::prepare_with(d_update, d_data) and
-    // compress_add_update in one call; the threshold is left in d_thr_out (device).  Returns false,
-    // having done nothing, when the compressor has no such fused path.
-    virtual bool compress_topk_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update,
-                                      int n, float topK, VarTYPE* d_thr_out, int* d_size_prefix) {
+    // Not in the reference.  ThresholdTopK(rule)::prepare_with(d_update, d_data) and
+    // compress_add_update as one call that only enqueues work; the threshold is left in d_thr_out.
+    // Returns false, having done nothing, when the compressor has no such path.
+    virtual bool write_step_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
+                                   const typename ThresholdFunction<VarTYPE>::TopKRule& rule, VarTYPE* d_thr_out,
+                                   int* d_size_prefix) {
         return false;
     }
 
@@ -154,10 +155,12 @@ public:
                                   wait ? &bytes : nullptr));
         return bytes;
     }
-    virtual bool compress_topk_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update,
-                                      int n, float topK, VarTYPE* d_thr_out, int* d_size_prefix) {
-        cxx::check(cx_ip_compress_topk(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, d_target, capacity, d_data,
-                                       d_update, n, topK, d_thr_out, d_size_prefix, nullptr));
+    virtual bool write_step_device(void* d_target, long long capacity, const VarTYPE* d_data, VarTYPE* d_update, int n,
+                                   const typename ThresholdFunction<VarTYPE>::TopKRule& rule, VarTYPE* d_thr_out,
+                                   int* d_size_prefix) {
+        cxx::check(cx_ip_write_step(this->handle_.get(), cxx::dtype_of<VarTYPE>::value, d_target, capacity, d_data,
+                                    d_update, n, rule.topK, rule.default_subsamples, rule.subsample_factor,
+                                    rule.d_positions, rule.n_positions, d_thr_out, d_size_prefix, nullptr));
         return true;
     }
     virtual int decompress_device(VarTYPE* d_output, int output_size, const void* d_source, bool wait) {

@@ -206,6 +206,21 @@ int cx_ip_compress_topk(cx_handle h, cx_dtype dt, void* out_msg, long long out_c
                         const void* data, void* update, int n, float topK,
                         void* d_thr_out, int* d_size_prefix, int* h_bytes);
 
+/* ComprEx<T>::writeRemote with ANY ThresholdTopK (src/comprEx.tpp:183-185): ThresholdTopK(topK,
+ * default_subsamples, subsample_factor)::prepare_with(update, data) (src/threshold.hxx:160-167,
+ * 182-240: the whole vector when n < subsamples, else `subsamples` strided positions) followed by
+ * compress_add_update with that threshold, as one call.  d_idx / m (device int32 positions, m > 0)
+ * replace the strided rule by the caller's sample positions.  A whole-vector threshold takes
+ * cx_ip_compress_topk's route, a sampled one cx_topk_threshold[_indexed] + cx_ip_compress: the same
+ * kernels, message, residual and threshold as the separate calls, enqueued by one call that never
+ * waits unless asked to (so that a caller may capture it in a HIP graph: short vectors are all
+ * launch latency, and a replayed graph halves it).  The threshold is left in d_thr_out (device T;
+ * NULL = the handle's slot).  h_bytes != NULL waits and returns the byte count. */
+int cx_ip_write_step(cx_handle h, cx_dtype dt, void* out_msg, long long out_capacity,
+                     const void* data, void* update, int n, float topK, int default_subsamples,
+                     float subsample_factor, const int* d_idx, int m, void* d_thr_out,
+                     int* d_size_prefix, int* h_bytes);
+
 /* CompressorRLE<T> (src/compressor.hxx:158-532), the run-length codec: message
  * int32 n | int32 c | c values | int32 runs | int32 signum | runs x int32 run lengths, an element
  * is sent when |x| >= threshold.  cx_rle_compress = compression_strategy (:167-390) in its three

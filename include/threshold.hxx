@@ -67,6 +67,17 @@ public:
     // and message in one fused call and leaves the threshold where claim_device_threshold() says.
     virtual bool whole_vector_topk(int n, float* topK_out) const { return false; }
     virtual VarTYPE* claim_device_threshold() { return nullptr; }
+    // Not in the reference.  The parameters of a top-k threshold (fraction, sub-sampling rule, optional
+    // caller-chosen sample positions on the device), for a caller that runs prepare_with and the
+    // compression as one call; false for every other kind of threshold.
+    struct TopKRule {
+        float topK;
+        int default_subsamples;
+        float subsample_factor;
+        const int* d_positions;
+        int n_positions;
+    };
+    virtual bool topk_rule(TopKRule*) const { return false; }
 
 protected:
     virtual bool is_aboveThreshold(const VarTYPE& target) = 0;
@@ -189,6 +200,14 @@ public:
         const int subsamples = cx_topk_subsamples(topK, default_subsamples, subsamples_factor);
         if (topK_out) *topK_out = topK;
         return subsamples < 0 || n < subsamples;
+    }
+    virtual bool topk_rule(typename ThresholdFunction<VarTYPE>::TopKRule* rule) const {
+        rule->topK = topK;
+        rule->default_subsamples = default_subsamples;
+        rule->subsample_factor = subsamples_factor;
+        rule->d_positions = sample_m_ > 0 ? static_cast<const int*>(sample_idx_.data()) : nullptr;
+        rule->n_positions = sample_m_;
+        return true;
     }
     // the slot will hold the threshold once the caller's fused call has run
     virtual VarTYPE* claim_device_threshold() {
