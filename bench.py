@@ -123,6 +123,120 @@ def cpu_reduce_baseline(msgs_h, n, seconds):
     return float(np.median(red)) * 1e3, float(np.median(app)) * 1e3, impl.kind, len(red)
 
 
+def golden_rows(name):
+    """Recorded outputs of the compiled reference for a configuration (tests/golden/full_size.json,
+    written by tests/golden/make_golden.py), or [] when the file is not there."""
+    try:
+        return json.load(open(os.path.join(ROOT, "tests", "golden", "full_size.json"))).get(name, [])
+    except (OSError, ValueError):
+        return []
+
+
+def config_leg(torch, W, cfg, grad_fn, cpu_seconds, with_cpu, cpu_iters_cap):
+    """One of the smaller configurations (C1, C2, C3): exact top-k threshold + fused compress per
+    iteration, residual carried, as ONE call per iteration (cx_ip_write_step: what
+    ComprEx::writeRemote enqueues).  Timed eagerly (events around every call) and, where the call
+    never waits, as a replayed HIP graph of `ring` iterations (short vectors are launch latency:
+    the graph removes the host's share of it).  The first iterations are compared bit for bit with
+    the compiled reference's recorded outputs."""
+    from comprex_amd.device import Handle, message_capacity
+    n, topk, ds = cfg["n"], np.float32(cfg["topK"]), cfg["default_subsamples"]
+    ring = 4
+    grads_h = [grad_fn(it) for it in range(ring)]
+    side = torch.cuda.Stream()
+    out = {"workload": cfg["name"], "n": n, "topK": float(topk)}
+    with torch.cuda.stream(side):
+        h = Handle()
+        grads = [torch.from_numpy(g).cuda() for g in grads_h]
+        rests = torch.zeros(n, device="cuda")
+        msg = torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+        hdr = msg[:8].view(torch.int32)
+
+        # parity: the recorded reference outputs of the first iterations
+        rows = golden_rows(cfg["name"].split("-")[0])
+        checked = 0
+        for it in range(ring):
+            nbytes = h.write_step(msg, grads[it], rests, topk, ds)
+            if it < len(rows) and rows[it].get("input") == W.checksum(grads_h[it]):
+                m_h = msg[:nbytes].cpu().numpy()
+                assert int(hdr[1].item()) == rows[it]["k"] and W.checksum(m_h) == rows[it]["msg"], \
+                    "%s iteration %d differs from the reference's recorded message" % (cfg["name"], it)
+                assert W.checksum(rests.cpu().numpy()) == rows[it]["rests"]
+                checked += 1
+        out["iterations_checked_against_reference"] = checked
+        fused_route = h.get_option("fused_topk_taken")  # 1: single pass over the vectors (waits once per call)
+
+        def step(it):
+            h.write_step(msg, grads[it % ring], rests, topk, ds, sync=False)
+
+        reps = 10 * ring
+        for it in range(2 * ring):
+            step(it)
+        side.synchronize()
+        e0 = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+        e1 = [torch.cuda.Event(enable_timing=True) for _ in range(reps)]
+        ks = []
+        for it in range(reps):
+            e0[it].record(side)
+            step(it)
+            e1[it].record(side)
+        side.synchronize()
+        eager_us = float(np.median([a.elapsed_time(b) for a, b in zip(e0, e1)])) * 1e3
+        k = int(hdr[1].item())
+        step_bytes = 20 * n + 8 * k + 8
+        out.update(k_last=k, algorithmic_bytes=step_bytes, eager_us=eager_us,
+                   eager_GBps=step_bytes / (eager_us * 1e-6) / 1e9,
+                   eager_frac=step_bytes / (eager_us * 1e-6) / 1e9 / HBM_PEAK_GBPS)
+        if fused_route == 0:
+            # the call only enqueues: capture `ring` iterations, replay them back to back
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for it in range(ring):
+                    step(it)
+            side.synchronize()
+            for _ in range(3):
+                graph.replay()
+            side.synchronize()
+            g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            replays = 20
+            g0.record(side)
+            for _ in range(replays):
+                graph.replay()
+            g1.record(side)
+            side.synchronize()
+            graph_us = g0.elapsed_time(g1) * 1e3 / (replays * ring)
+            out.update(graph_us=graph_us, graph_GBps=step_bytes / (graph_us * 1e-6) / 1e9,
+                       graph_frac=step_bytes / (graph_us * 1e-6) / 1e9 / HBM_PEAK_GBPS)
+            del graph
+        else:
+            out["graph_us"] = None  # the single-pass route reads one word back per call: not capturable
+        h.synchronize()
+        h.close()
+    log("%s: step %.1f us eager%s (%.0f GB/s of 20n+8k+8, %.1f%% of peak), k=%d, %d iterations checked"
+        % (cfg["name"], eager_us, "" if out.get("graph_us") is None else ", %.1f us as a replayed graph" % out["graph_us"],
+           out["eager_GBps"], 100 * out["eager_frac"], k, checked))
+    if with_cpu:
+        from oracle.pyoracle import Oracle, ref_available
+        impl = Oracle(ref=True) if ref_available() else Oracle()
+        rests_h = np.zeros(n, np.float32)
+        times = []
+        t_end = time.perf_counter() + cpu_seconds
+        it = 0
+        while it < 2 or (time.perf_counter() < t_end and it < cpu_iters_cap):
+            g = grads_h[it % ring]
+            t0 = time.perf_counter()
+            thr = impl.calc_threshold(rests_h + g, topk)   # prep_add_vec (whole vector) + nth_element
+            impl.ip_compress(g, rests_h, thr)               # compress_add_update
+            if it > 0:
+                times.append(time.perf_counter() - t0)
+            it += 1
+        med = float(np.median(times))
+        out["cpu_baseline"] = {"cores": 1, "kind": impl.kind, "us": med * 1e6, "GBps": step_bytes / med / 1e9,
+                               "sample": "%d iterations after 1 warm-up, median" % len(times)}
+        log("%s cpu baseline (%s, 1 core): %.0f us/iteration" % (cfg["name"], impl.kind, med * 1e6))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +249,8 @@ def main():
     ap.add_argument("--items", type=int, default=None, help="compaction tile option (2/4/8)")
     ap.add_argument("--alternate", type=int, default=None, help="stage_alternate option (0/1)")
     ap.add_argument("--cached-tail-mb", type=int, default=None, help="stage_cached_tail_mb option (-1 = all cacheable)")
+    ap.add_argument("--configs-only", action="store_true",
+                    help="run only the legs of the smaller configurations C1, C2, C3 (for a kernel trace of them)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of the gradient (4n bytes read, 4n written) so that "
                          "a counter run has a kernel of known traffic to scale FETCH_SIZE/WRITE_SIZE by")
@@ -149,6 +265,13 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.configs_only:
+        legs = {}
+        for key, cfg, fn, cap in (("C1", W.C1, W.c1_gradient, 100), ("C2", W.C2, W.c2_gradient, 200),
+                                  ("C3", W.C3, W.c3_gradient, 3)):
+            legs[key] = config_leg(torch, W, cfg, fn, min(args.cpu_seconds, 5.0), not args.no_cpu, cap)
+        print(json.dumps({"configs": legs}), flush=True)
+        return
     n = args.n or W.C4["n"]
     topk = np.float32(W.C4["topK"])
     m = W.C4["n_samples"] if n >= W.C4["n_samples"] * 10 else max(1000, n // 100)
@@ -312,6 +435,16 @@ def main():
         del g, rests, msg
         torch.cuda.empty_cache()
 
+        if n == W.C4["n"]:
+            # the other compress configurations, each as its own leg
+            extra["configs"] = {}
+            for key, cfg, fn, cap in (("C1", W.C1, W.c1_gradient, 100), ("C2", W.C2, W.c2_gradient, 200),
+                                      ("C3", W.C3, W.c3_gradient, 3)):
+                extra["configs"][key] = config_leg(torch, W, cfg, fn, min(args.cpu_seconds, 5.0), not args.no_cpu, cap)
+            extra["configs"]["launches_per_step"] = {
+                "C1": 6, "C2": 4, "C3": 9,
+                "source": "rocprofv3 kernel trace of these legs, profiles/configs_C1_C2_C3_kernel_trace.txt, not this run"}
+
         # reduce: 8 simulated ranks' 1 %-dense messages into a 64 Mi dense vector (config C5)
         c5n = W.C5["n"] if n == W.C4["n"] else 1 << 22
         c5k = W.C5["k"] if n == W.C4["n"] else c5n // 100
@@ -345,6 +478,34 @@ def main():
                                 "frac": acc_bytes / (acc_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
         log("reduce ordered, added into the vector %.3f ms (%.0f GB/s of 8n+16Rk, %.1f%% of peak)"
             % (acc_ms, reduce["accumulate"]["GBps"], 100 * reduce["accumulate"]["frac"]))
+        # The chief's apply as the reference runs it (src/allreduce.tpp:183-205): readRemote_add per
+        # worker into its own vector (here ONE rank-ordered accumulate), then the broadcast leg's
+        # writeRemote(data): residual += reduced vector, exact top-k 1 %, compact, zero
+        c5_brests = torch.zeros(c5n, device="cuda")
+        bmsg = torch.zeros(8 + 8 * (c5n // 25), dtype=torch.uint8, device="cuda")
+        ds_exact = 1 << 27 if c5n >= 1 << 23 else 1 << 30
+
+        def chief_apply():
+            h.reduce(dense, msgs, accumulate=True, mode=0)
+            h.write_step(bmsg, dense, c5_brests, np.float32(0.01), ds_exact)  # (the single pass waits once)
+
+        for _ in range(2):
+            chief_apply()
+        ca_ms = event_ms(torch, chief_apply, reps)
+        kb = int(bmsg[4:8].view(torch.int32).item())
+        ca_bytes = acc_bytes + 12 * c5n + 8 * kb + 8
+        for _ in range(2):
+            h.write_step(bmsg, dense, c5_brests, np.float32(0.01), ds_exact)
+        bw_ms = event_ms(torch, lambda: h.write_step(bmsg, dense, c5_brests, np.float32(0.01), ds_exact), reps)
+        reduce["chief_apply"] = {"what": "accumulating rank-ordered reduce into the chief's vector, then writeRemote of it "
+                                         "(exact top-k 1 %) on the broadcast channel",
+                                 "algorithmic_bytes": ca_bytes, "ms": ca_ms, "GBps": ca_bytes / (ca_ms * 1e-3) / 1e9,
+                                 "frac": ca_bytes / (ca_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                                 "broadcast_leg_alone_ms": bw_ms, "reduce_alone_ms": acc_ms, "k_broadcast": kb}
+        log("chief's apply (accumulate + broadcast-leg writeRemote): %.3f ms (%.0f GB/s of 8n+16Rk+12n+8k, %.1f%% of peak); "
+            "parts alone %.3f + %.3f ms" % (ca_ms, reduce["chief_apply"]["GBps"], 100 * reduce["chief_apply"]["frac"],
+                                            acc_ms, bw_ms))
+        del c5_brests, bmsg
         # residual apply (K4): rests += dense, 12 bytes per element
         c5_rests = torch.zeros(c5n, device="cuda")
         for _ in range(2):
@@ -394,6 +555,14 @@ def main():
                      "traffic_source": "committed counter run profiles/stage_kernel_C4_100M_pmc.txt, not this run",
                      "kernel": "stage_kernel<float,0,4,%d>" % (args.items or 4), "algorithmic_bytes": kern_bytes,
                      "avg_ms": kern_ms, "cache_state": "warm (see extra.cold for the cold-residual figures)"},
+        "roofline_realistic": {"bound": "hbm", "achieved": extra["gradient_rewritten"]["stage_kernel_GBps"],
+                               "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": extra["gradient_rewritten"]["stage_kernel_frac"],
+                               "kernel": "stage_kernel<float,0,4,%d>" % (args.items or 4), "algorithmic_bytes": kern_bytes,
+                               "avg_ms": extra["gradient_rewritten"]["stage_kernel_ms"],
+                               "step_frac": extra["gradient_rewritten"]["hbm_peak_fraction_step"],
+                               "cache_state": "the gradient is rewritten in place by another kernel between two steps, as a "
+                                              "backward pass leaves it: the memory-side cache holds its dirty tail, not the "
+                                              "residual's"},
         "cpu_baseline": cpu,
         "extra": extra,
     }
