@@ -35,19 +35,18 @@ namespace cx {
 
 namespace {
 
-#ifndef CX_STAGE_BLOCK
-#define CX_STAGE_BLOCK 256
-#endif
-constexpr int kBlock = CX_STAGE_BLOCK;  // threads of a streaming block: one tile per wavefront
+// threads of a streaming block, one tile per wavefront.  Measured on 100 M fp32 elements at 1 %, whole
+// step: 128 / 256 / 512 threads 0.210 / 0.208 / 0.209 ms back to back and 0.223 / 0.222 / 0.221 ms after
+// the gradient was rewritten, i.e. alike within the spread between two runs (0.001 ms).
+constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
-#ifndef CX_GATHER_UNROLL
-#define CX_GATHER_UNROLL 4
-#endif
-#ifndef CX_GATHER_BLOCK
-#define CX_GATHER_BLOCK 256
-#endif
-constexpr int kGatherBlock = CX_GATHER_BLOCK;  // threads of a gather block
+// threads of a gather block and pairs a lane moves per round.  Measured, whole step as above: 128 / 256 /
+// 512 threads and 2 / 4 / 8 pairs all give 0.208 ms (0.222-0.223 ms after the gradient was rewritten); on
+// 61 706 elements at 10 % the threshold + compress take 50 / 42 / 41 us with 128 / 256 / 512 threads and
+// 44 / 42 / 42 us with 2 / 4 / 8 pairs.
+constexpr int kGatherBlock = 256;
+constexpr int kGatherUnroll = 4;
 constexpr int kGatherTiles = 64;                // tiles a gather block owns: one lane per tile in its scan
 static_assert(kGatherTiles % (kWavesPerBlock * 8) == 0, "a gather block's streaming blocks fill whole 16-byte loads of 16-bit sums");
 static_assert(kWavesPerBlock * 64 * 4 * 16 <= 65535, "a streaming block's survivors fit 16 bits (largest tile: 64 lanes x 16 loads x 4 elements)");
@@ -63,12 +62,10 @@ template <typename T, int V> struct alignas(sizeof(T) * V) Pack { T x[V]; };
 // elements (step, everything cacheable -> 192 MB tail): consecutive steps 0.214 -> 0.206 ms; after
 // another kernel read 1 GiB 0.218 -> 0.214 ms, rewrote 1 GiB 0.265 -> 0.248 ms, rewrote the
 // gradient itself 0.250 -> 0.221 ms.  (No cacheable reads at all: 0.221 / 0.223 / 0.232 / 0.224 ms.)
-#ifndef CX_NT_DATA
-#define CX_NT_DATA 1
-#endif
-#ifndef CX_NT_UPDATE_STORE
-#define CX_NT_UPDATE_STORE 1
-#endif
+// (the same step with cacheable gradient loads: 0.208 -> 0.226 ms, after the gradient was rewritten
+// 0.222 -> 0.267 ms; with cacheable residual stores: 0.229 and 0.253 ms)
+constexpr bool kNontemporalData = true;         // gradient loads
+constexpr bool kNontemporalUpdateStore = true;  // residual stores
 
 template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p, bool nt) {
@@ -155,7 +152,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         for (int j = 0; j < ITEMS; ++j) {
             const long long e0 = base + (long long)j * (64 * VEC) + (long long)lane * VEC;
             if (MODE != 2) uu[j] = load_pack<T, VEC>(update + e0, nt_update);
-            if (MODE != 1) dd[j] = load_pack<T, VEC>(data + e0, CX_NT_DATA != 0);
+            if (MODE != 1) dd[j] = load_pack<T, VEC>(data + e0, kNontemporalData);
             valid_mask[j] = (1u << VEC) - 1u;
         }
     } else {
@@ -241,7 +238,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         }
         if (MODE != 2) {
             if (full) {
-                if (MODE == 0 || MODE == 3 || m != 0u) store_pack<T, VEC>(update + e0, w, CX_NT_UPDATE_STORE != 0);
+                if (MODE == 0 || MODE == 3 || m != 0u) store_pack<T, VEC>(update + e0, w, kNontemporalUpdateStore);
             } else {
 #pragma unroll
                 for (int c = 0; c < VEC; ++c)
@@ -331,28 +328,15 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
     constexpr int kWaves = kGatherBlock / 64;
     // pairs a lane moves per round: searches and loads of one round are independent
-    constexpr int kCopyUnroll = CX_GATHER_UNROLL;
+    constexpr int kCopyUnroll = kGatherUnroll;
     __shared__ unsigned s_before[kWaves];
     __shared__ unsigned s_off[65];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    unsigned before = 0;
-    {
-        // stage blocks before this block's first tile: kGatherTiles / kWavesPerBlock per gather block
-        // (eight 16-bit sums per 16-byte load)
-        const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
-        const unsigned nvec = blockIdx.x * (kGatherTiles / kWavesPerBlock / 8);
-#pragma unroll 8
-        for (unsigned v = tid; v < nvec; v += kGatherBlock) {
-            const uint4 c = b4[v];
-            before += (c.x & 0xffffu) + (c.x >> 16) + (c.y & 0xffffu) + (c.y >> 16) + (c.z & 0xffffu) + (c.z >> 16) +
-                      (c.w & 0xffffu) + (c.w >> 16);
-        }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
-    if (lane == 0) s_before[wave] = before;
-
+    // Order of the loads: the tiles' counts first, then (their scan known) the staged pairs of the first
+    // round, and only then the sums of the streaming blocks before this block's tiles, which give the
+    // pairs' destination: the long read of the sums runs while the staged pairs are on their way,
+    // instead of in front of everything (a memory round trip or two less on a kernel that is all latency).
     // every wavefront scans the same 64 counts
     const unsigned first = blockIdx.x * kGatherTiles;
     const unsigned tile = first + lane;  // tiles past the end count as empty
@@ -370,6 +354,51 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
         if (lane == 63) s_off[64] = block_pairs;
     }
     const unsigned long long deferred = __ballot((raw & kDeferred) != 0u);
+    __syncthreads();
+
+    // one round of the copy: where a pair of this block comes from (its tile's slot) and its words
+    unsigned src_idx[kCopyUnroll];
+    bool live[kCopyUnroll];
+    unsigned v[kCopyUnroll][PW];
+    auto load_round = [&](unsigned p0) {
+#pragma unroll
+        for (int q = 0; q < kCopyUnroll; ++q) {
+            const unsigned p = p0 + q * kGatherBlock + tid;
+            live[q] = p < block_pairs;
+            // owner: last tile of this block whose exclusive offset is <= p.  Six fixed steps
+            // without branches, so that the searches of one round overlap their LDS reads.
+            int lo = 0;
+#pragma unroll
+            for (int step = 32; step > 0; step >>= 1)
+                lo += (s_off[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
+            if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
+            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - s_off[lo]);
+        }
+#pragma unroll
+        for (int q = 0; q < kCopyUnroll; ++q)
+            if (live[q]) {
+#pragma unroll
+                for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
+            }
+    };
+    load_round(0u);
+
+    unsigned before = 0;
+    {
+        // stage blocks before this block's first tile: kGatherTiles / kWavesPerBlock per gather block
+        // (eight 16-bit sums per 16-byte load)
+        const uint4* b4 = reinterpret_cast<const uint4*>(block_sums);
+        const unsigned nvec = blockIdx.x * (kGatherTiles / kWavesPerBlock / 8);
+#pragma unroll 8
+        for (unsigned i = tid; i < nvec; i += kGatherBlock) {
+            const uint4 c = b4[i];
+            before += (c.x & 0xffffu) + (c.x >> 16) + (c.y & 0xffffu) + (c.y >> 16) + (c.z & 0xffffu) + (c.z >> 16) +
+                      (c.w & 0xffffu) + (c.w >> 16);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off, 64);
+    if (lane == 0) s_before[wave] = before;
     __syncthreads();
     unsigned block_base = 0;
 #pragma unroll
@@ -391,28 +420,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     unsigned* const pairs = msg_words + 2;
     bool overflow = false;
     for (unsigned p0 = 0; p0 < block_pairs; p0 += kGatherBlock * kCopyUnroll) {
-        unsigned src_idx[kCopyUnroll];
-        bool live[kCopyUnroll];
-#pragma unroll
-        for (int q = 0; q < kCopyUnroll; ++q) {
-            const unsigned p = p0 + q * kGatherBlock + tid;
-            live[q] = p < block_pairs;
-            // owner: last tile of this block whose exclusive offset is <= p.  Six fixed steps
-            // without branches, so that the searches of one round overlap their LDS reads.
-            int lo = 0;
-#pragma unroll
-            for (int step = 32; step > 0; step >>= 1)
-                lo += (s_off[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
-            if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
-            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - s_off[lo]);
-        }
-        unsigned v[kCopyUnroll][PW];
-#pragma unroll
-        for (int q = 0; q < kCopyUnroll; ++q)
-            if (live[q]) {
-#pragma unroll
-                for (int w = 0; w < PW; ++w) v[q][w] = staging[(long long)src_idx[q] * PW + w];
-            }
+        if (p0 > 0u) load_round(p0);
 #pragma unroll
         for (int q = 0; q < kCopyUnroll; ++q)
             if (live[q]) {

@@ -72,16 +72,17 @@ __global__ __launch_bounds__(kBlock) void select_final_kernel(SelectState* st, u
 }
 
 // One histogram pass over the keys described by (vec, add, idx).  SMODE: 0 whole vector,
-// 1 strided, 2 indexed.
+// 1 strided, 2 indexed.  The first `nblocks` blocks of the grid share the keys; the others leave.
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
-__global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
-                                                             const int* __restrict__ idx, long long m, int n,
-                                                             float stepsize, SelectState* __restrict__ st, int p,
-                                                             unsigned long long rank0) {
+__device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __restrict__ add,
+                                          const int* __restrict__ idx, long long m, int n, float stepsize,
+                                          SelectState* __restrict__ st, int p, unsigned long long rank0,
+                                          unsigned nblocks) {
     using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
     __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    if (blockIdx.x >= nblocks) return;
     // chained passes: every block redoes the cheap pick over the previous pass's complete histogram
     PickState s;
     s.prefix = 0ull;
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
     int shift, bits;
     pass_digits_dev<T>(p, shift, bits);
     const unsigned digit_mask = (1u << bits) - 1u;
-    const long long stride = (long long)gridDim.x * kBlock;
+    const long long stride = (long long)nblocks * kBlock;
 
     if (SMODE == 0 && VEC > 1) {
         const long long nvec = m / VEC;
@@ -149,6 +150,38 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
     for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
         const unsigned c = lds_hist[b];
         if (c) atomicAdd(&st->pass_hist[p][b], c);
+    }
+}
+
+template <typename T, int SMODE, bool HAS_ADD, int VEC>
+__global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                             const int* __restrict__ idx, long long m, int n,
+                                                             float stepsize, SelectState* __restrict__ st, int p,
+                                                             unsigned long long rank0) {
+    hist_pass<T, SMODE, HAS_ADD, VEC>(vec, add, idx, m, n, stepsize, st, p, rank0, gridDim.x);
+}
+
+// The same pass where the DEVICE decides what is counted: the *cand_count candidate keys (magnitude bit
+// patterns, i.e. a vector of |x|) when they hold the wanted rank and all fit their buffer, the whole
+// vector(s) otherwise.  Every pass of a selection reads the same count and decides alike, so the
+// host launches the passes without knowing which way they go.  The grid is sized for the whole
+// vector; over the candidates only the blocks they need stay.
+template <typename T, bool HAS_ADD, int VEC>
+__global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                                    long long m,
+                                                                    const typename Elem<T>::key_t* __restrict__ cand,
+                                                                    unsigned cap, const unsigned* __restrict__ cand_count,
+                                                                    SelectState* __restrict__ st, int p,
+                                                                    unsigned long long rank0) {
+    const unsigned count = *cand_count;
+    if ((unsigned long long)count > rank0 && count <= cap) {
+        constexpr unsigned kPerBlock = (unsigned)kBlock * VEC * 8u;
+        unsigned need = (count + kPerBlock - 1u) / kPerBlock;
+        if (need > gridDim.x) need = gridDim.x;
+        hist_pass<T, 0, false, VEC>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
+                                    st, p, rank0, need);
+    } else {
+        hist_pass<T, 0, HAS_ADD, VEC>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
     }
 }
 
@@ -232,10 +265,10 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
 // device-wide release per block and an acquire in the last one, and on this GPU those write back
 // and invalidate the L2 of the block's XCD (0.5 to 1.2 us and 2.5 us; 30 us more with a fence in
 // every thread), which is what the launch boundary does anyway.
-#ifndef CX_FIRST_BLOCK
-#define CX_FIRST_BLOCK 1024
-#endif
-constexpr int kFirstBlock = CX_FIRST_BLOCK;  // threads per block of the first launch, one key each
+// threads per block of the first launch, one key each.  Measured, threshold + compress: 256 / 512 / 1024
+// threads give 0.213 / 0.207 / 0.208 ms on 100 M elements with 100 000 sampled positions and 39 / 44 / 42 us
+// on all of 61 706 elements.
+constexpr int kFirstBlock = 1024;
 constexpr int kFinishBlock = 1024;
 constexpr int kListBytes = 49152;           // LDS list of the last block
 constexpr int kShortGlobalKeys = 1 << 16;   // capacity of the short list in device memory
@@ -394,7 +427,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
                                                                      unsigned long long rank, int plus_one,
                                                                      T* __restrict__ thr_out, int short_on,
                                                                      const typename Elem<T>::key_t* __restrict__ short_keys,
-                                                                     unsigned short_cap) {
+                                                                     unsigned short_cap, unsigned* __restrict__ zero_word) {
     using key_t = typename Elem<T>::key_t;
     constexpr int kKeyBits = Elem<T>::key_bits;
     constexpr int kListKeys = kListBytes / (int)sizeof(key_t);
@@ -423,6 +456,7 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
         st->short_count = 0u;
         st->short_digit = 0u;
     }
+    if (zero_word && t == 0) *zero_word = 0u;  // a counter the kernels after this one start from
     key_t prefix = 0, mask = 0;
     int lo = kKeyBits;  // the bits below this one are still open
     // where the keys still in play are read from: the key array, the short list, or (listed) LDS
@@ -569,18 +603,14 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
 // Copies every key >= the key of *d_bound into `cand` (order irrelevant).  Each wavefront
 // gathers its matches in an LDS segment and appends the segment with ONE global atomic when it
 // fills up and at the end, so the counter sees a few thousand atomics per pass, not one per hit.
-// *cand_count keeps counting past `cap`; the host falls back when it overflows.
-// Cache policy of the one-pass candidate collection, as in the streaming pass of the compress: the
-// gradient (bit 1) bypasses the caches, the residual (bit 0) stays cacheable.  Measured on 100 M
-// fp32 elements, threshold + compress as two calls: 0.436 ms with plain loads, 0.404 ms with either
-// vector or both nontemporal.
-#ifndef CX_COLLECT_NT
-#define CX_COLLECT_NT 2
-#endif
-#ifndef CX_COLLECT_UNROLL
-#define CX_COLLECT_UNROLL 4
-#endif
-constexpr int kCollectUnroll = CX_COLLECT_UNROLL;  // 16-byte loads in flight per lane
+// *cand_count keeps counting past `cap`; the passes that follow see it and take the whole vector(s) instead.
+// Cache policy of the one-pass candidate collection: both vectors bypass the caches.  Measured on 100 M
+// fp32 elements, threshold alone / threshold + compress as two calls: both nontemporal 0.165 / 0.360 ms,
+// the gradient only 0.168 / 0.373 ms, neither 0.178 / 0.403 ms.  16-byte loads in flight per lane:
+// 2 / 4 / 8 give 0.196 / 0.168 / 0.171 ms for the threshold alone.
+constexpr bool kCollectNontemporalVec = true;    // first vector (the residual, when there are two)
+constexpr bool kCollectNontemporalAdd = true;   // second vector (the gradient)
+constexpr int kCollectUnroll = 4;               // 16-byte loads in flight per lane
 // every wavefront ends with one returning atomic on the one counter, and those queue up: measured on
 // 100 M elements, 256 / 512 / 1024 / 2048 / 4096 blocks take 0.252 / 0.207 / 0.218 / 0.243 / 0.306 ms
 constexpr int kCollectBlocks = 512;
@@ -642,19 +672,14 @@ __global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restr
             in[u] = g >= 0 && i < nvec;
             if (in[u]) {
                 typedef T vec_t __attribute__((ext_vector_type(VEC)));
-#if CX_COLLECT_NT & 1
-                const vec_t va = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(vec) + i);
-#else
-                const vec_t va = reinterpret_cast<const vec_t*>(vec)[i];
-#endif
+                const vec_t va = kCollectNontemporalVec ? __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(vec) + i)
+                                                        : reinterpret_cast<const vec_t*>(vec)[i];
 #pragma unroll
                 for (int c = 0; c < VEC; ++c) a[u].x[c] = va[c];
                 if (HAS_ADD) {
-#if CX_COLLECT_NT & 2
-                    const vec_t vb = __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(add) + i);
-#else
-                    const vec_t vb = reinterpret_cast<const vec_t*>(add)[i];
-#endif
+                    const vec_t vb = kCollectNontemporalAdd
+                                         ? __builtin_nontemporal_load(reinterpret_cast<const vec_t*>(add) + i)
+                                         : reinterpret_cast<const vec_t*>(add)[i];
 #pragma unroll
                     for (int c = 0; c < VEC; ++c) b[u].x[c] = vb[c];
                 }
@@ -768,7 +793,7 @@ inline size_t candidate_capacity(long long m) {
 
 template <typename T>
 int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d_idx, int m, int sample_mode,
-                float stepsize, unsigned long long rank, int plus_one, T* d_thr_out) {
+                float stepsize, unsigned long long rank, int plus_one, T* d_thr_out, unsigned* zero_word = nullptr) {
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     using key_t = typename Elem<T>::key_t;
 
@@ -801,10 +826,11 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
 #undef CX_FIRST_MODE
 #undef CX_FIRST
         hipLaunchKernelGGL(select_finish_kernel<T>, dim3(1), dim3(kFinishBlock), 0, h->stream, keys, m, h->sel, rank,
-                           plus_one, d_thr_out, short_k > 0 ? 1 : 0, short_keys, short_cap);
+                           plus_one, d_thr_out, short_k > 0 ? 1 : 0, short_keys, short_cap, zero_word);
         CX_HIP(hipGetLastError());
         return CX_OK;
     }
+    if (zero_word) return fail(CX_ERR_INTERNAL, "select: only the two-launch path clears a counter");
 
     const bool vec_ok =
         ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
@@ -823,14 +849,17 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
 // Whole-vector selection in ONE pass over the vector(s) when the wanted rank is near the top:
 //   1. a strided sample gives a lower bound L that, with overwhelming probability, has at
 //      least rank+1 keys at or above it, and not many more;
-//   2. one pass copies the keys >= L into a candidate buffer;
-//   3. the host reads the candidate count (the only synchronisation); when rank < count <= capacity
-//      the answer is the key of the same rank among the candidates, found on that small set.
-// Otherwise *done stays 0 and the caller runs the full three-pass selection.  Exact either way.
+//   2. one pass copies the keys >= L into a candidate buffer and counts them;
+//   3. chained radix passes whose blocks read that count: when rank < count <= capacity they run
+//      over the candidates (the answer is the key of the same rank among them), otherwise (bound too
+//      high, or ties flooded the buffer) over the whole vector(s).  Exact either way, and the host
+//      never waits: the call is asynchronous like the others.
+// Sets *done when the selection was launched; leaves it 0 when the path does not apply.
 template <typename T>
 int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, unsigned long long rank, int plus_one,
                           T* d_thr_out, int* done) {
     using key_t = typename Elem<T>::key_t;
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     *done = 0;
     constexpr int kSample = 1 << 16;
     const double p = (double)(rank + 1) / (double)m;
@@ -842,16 +871,17 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     const size_t cap = candidate_capacity(m);
     int rc_cand = ensure_candidates(h, cap * sizeof(key_t));
     if (rc_cand != CX_OK) return rc_cand;
-    // 1. lower bound from the sample, left in the second half of the threshold slot
+    // 1. lower bound from the sample, left in the second half of the threshold slot; the kernel that
+    //    writes it also clears the candidate counter
     T* d_bound = reinterpret_cast<T*>(static_cast<char*>(h->d_thr) + 64);
     unsigned* d_count = reinterpret_cast<unsigned*>(static_cast<char*>(h->d_thr) + 128);
     const float stepsize = (float)m / (float)kSample;
-    int rc = select_rank<T>(h, vec, add_vec, m, nullptr, kSample, kSampleStrided, stepsize, sample_rank, 0, d_bound);
+    int rc = select_rank<T>(h, vec, add_vec, m, nullptr, kSample, kSampleStrided, stepsize, sample_rank, 0, d_bound,
+                            d_count);
     if (rc != CX_OK) return rc;
     // 2. candidates; the pass starts at the end of the vectors where the previous pass stopped
     const int reverse = h->stage_alternate ? (int)h->parity : 0;
     h->parity ^= 1u;  // the next full pass (the compress that follows) walks the other way
-    CX_HIP(hipMemsetAsync(d_count, 0, sizeof(unsigned), h->stream));
     constexpr int kVec = 16 / (int)sizeof(T);
     key_t* cand = static_cast<key_t*>(h->cand);
     if (add_vec)
@@ -860,17 +890,22 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     else
         hipLaunchKernelGGL((select_collect_kernel<T, false, kVec>), dim3(kCollectBlocks), dim3(kBlock), 0, h->stream, vec,
                            add_vec, (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse);
+    // 3. the passes, over whichever the count allows
+    const long long per_block = (long long)kBlock * kVec * 8;
+    long long blocks = ((long long)m + per_block - 1) / per_block;
+    if (blocks > 2048) blocks = 2048;
+    for (int q = 0; q < kPasses; ++q) {
+        if (add_vec)
+            hipLaunchKernelGGL((select_hist_either_kernel<T, true, kVec>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
+                               vec, add_vec, (long long)m, cand, (unsigned)cap, d_count, h->sel, q, rank);
+        else
+            hipLaunchKernelGGL((select_hist_either_kernel<T, false, kVec>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
+                               vec, add_vec, (long long)m, cand, (unsigned)cap, d_count, h->sel, q, rank);
+    }
+    hipLaunchKernelGGL(select_final_kernel<T>, dim3(1), dim3(kBlock), 0, h->stream, h->sel, rank, plus_one, d_thr_out);
     CX_HIP(hipGetLastError());
-    // 3. how many?
-    CX_HIP(hipMemcpyAsync(h->h_pinned + 12, d_count, sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
-    CX_HIP(hipStreamSynchronize(h->stream));
-    const unsigned long long count = (unsigned)h->h_pinned[12];
-    if (count <= rank || count > cap) return CX_OK;  // bound too high (or ties flooded the buffer): full selection
-    // magnitudes' bit patterns order like the magnitudes: the candidates are a vector of |x|
-    rc = select_rank<T>(h, reinterpret_cast<const T*>(cand), nullptr, (int)count, nullptr, (int)count, kSampleFull,
-                        1.0f, rank, plus_one, d_thr_out);
-    if (rc == CX_OK) *done = 1;
-    return rc;
+    *done = 1;
+    return CX_OK;
 }
 
 template <typename T>

@@ -59,6 +59,30 @@ def test_reserve_takes_the_scratch_up_front(oracle):
     rle = torch.zeros(16 + 8 * n + 8, dtype=torch.uint8, device="cuda")
     idx = _gpu(np.sort(rng.integers(0, n, 50_000)).astype(np.int32))
     dense = torch.zeros(n, device="cuda")
+    def calls(h, check):
+        thr = h.topk_threshold_indexed(r, g, idx, np.float32(0.01))
+        nbytes = h.compress(msg, g, r)
+        if check:
+            assert thr == oracle.topk_prepare_indexed(np.zeros(n, np.float32), g_h, idx.cpu().numpy(), np.float32(0.01))
+            want = oracle.ip_compress(g_h, np.zeros(n, np.float32), np.float32(thr))
+            assert msg[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+        h.decompress(dense, msg)
+        h.reduce(dense, [msg, msg], accumulate=False, mode=0)
+        h.reduce(dense, [msg, msg], accumulate=True, mode=0)
+        h.reduce(dense, [msg] * 4, accumulate=False, mode=0)
+        h.compress_topk(msg, g, r, np.float32(0.001))
+        assert h.get_option("fused_topk_taken") == 1   # the one-pass route, whose candidate list was reserved
+        h.rle_compress(rle, g, r, thr=np.float32(thr))
+        h.synchronize()
+        r.zero_()
+
+    # the runtime places a source file's kernels in device memory on the first launch of one of them:
+    # a first handle runs the same calls (growing its own buffers as it goes) and is closed again
+    warm = Handle()
+    try:
+        calls(warm, False)
+    finally:
+        warm.close()
     h = Handle()
     try:
         with pytest.raises(RuntimeError):
@@ -68,19 +92,7 @@ def test_reserve_takes_the_scratch_up_front(oracle):
         h.reserve(n, torch.float32, Handle.RESERVE_ALL)
         torch.cuda.synchronize()
         free_before = torch.cuda.mem_get_info()[0]
-        thr = h.topk_threshold_indexed(r, g, idx, np.float32(0.01))
-        assert thr == oracle.topk_prepare_indexed(np.zeros(n, np.float32), g_h, idx.cpu().numpy(), np.float32(0.01))
-        nbytes = h.compress(msg, g, r)
-        want_r = np.zeros(n, np.float32)
-        want = oracle.ip_compress(g_h, want_r, np.float32(thr))
-        assert msg[:nbytes].cpu().numpy().tobytes() == want.tobytes()
-        h.decompress(dense, msg)
-        h.reduce(dense, [msg, msg], accumulate=False, mode=0)
-        h.reduce(dense, [msg, msg], accumulate=True, mode=0)
-        h.compress_topk(msg, g, r, np.float32(0.001))
-        assert h.get_option("fused_topk_taken") == 1   # the one-pass route, whose candidate list was reserved
-        h.rle_compress(rle, g, r, thr=np.float32(thr))
-        h.synchronize()
+        calls(h, True)
         assert torch.cuda.mem_get_info()[0] == free_before
     finally:
         h.close()
