@@ -62,8 +62,9 @@ struct SelectState {
     unsigned int short_count;      // two-launch select: keys in the short list; zero between runs
     unsigned int short_digit;      // ... and the largest cut of a block: the leading two digits of its short_k-th key
     // chained passes (no pick launch in between): one histogram per pass, all zero between runs,
-    // and the state entering each pass
-    unsigned int pass_hist[kMaxRadixPasses][kRadixBins];
+    // and the state entering each pass.  The slot behind a key type's last pass holds the top-digit
+    // counts of a candidate list, made by the kernel that collects the list.
+    unsigned int pass_hist[kMaxRadixPasses + 1][kRadixBins];
     PickState pass_state[kMaxRadixPasses];
 };
 

@@ -90,12 +90,14 @@ template <typename T> __device__ __forceinline__ void pass_digits_dev(int p, int
 // st->pass_hist[p]; every block of the NEXT kernel redoes the cheap pick over it on its own
 // (a complete histogram is visible to all of them: it was finished by the previous kernel), so
 // no block ever waits for another and no launch is spent on a one-block kernel.
-// Returns the state entering pass p (p >= 1): the digits of passes 0..p-1 fixed.
+// Returns the state entering pass p (p >= 1): the digits of passes 0..p-1 fixed.  `prev_hist`
+// replaces pass p-1's histogram when those counts were made elsewhere.
 template <typename T, int BLOCK>
 __device__ __forceinline__ PickState state_entering_pass(const SelectState* __restrict__ st, int p,
                                                          unsigned long long rank0, unsigned* lds_hist,
                                                          unsigned long long* s_sum, unsigned* s_digit,
-                                                         unsigned long long* s_above) {
+                                                         unsigned long long* s_above,
+                                                         const unsigned* __restrict__ prev_hist = nullptr) {
     PickState s;
     if (p == 1) {
         s.prefix = 0ull;
@@ -104,7 +106,8 @@ __device__ __forceinline__ PickState state_entering_pass(const SelectState* __re
     } else {
         s = st->pass_state[p - 1];
     }
-    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) lds_hist[b] = st->pass_hist[p - 1][b];
+    const unsigned* counts = prev_hist ? prev_hist : st->pass_hist[p - 1];
+    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) lds_hist[b] = counts[b];
     __syncthreads();
     unsigned digit;
     unsigned long long above;

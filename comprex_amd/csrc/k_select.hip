@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kBlock) void select_final_kernel(SelectState* st, u
         if (plus_one) v = (T)(v + 1);
         *thr_out = v;
     }
-    for (int b = threadIdx.x; b < kPasses * kRadixBins; b += kBlock) (&st->pass_hist[0][0])[b] = 0u;
+    for (int b = threadIdx.x; b < (kPasses + 1) * kRadixBins; b += kBlock) (&st->pass_hist[0][0])[b] = 0u;
 }
 
 // One histogram pass over the keys described by (vec, add, idx).  SMODE: 0 whole vector,
@@ -77,7 +77,7 @@ template <typename T, int SMODE, bool HAS_ADD, int VEC>
 __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __restrict__ add,
                                           const int* __restrict__ idx, long long m, int n, float stepsize,
                                           SelectState* __restrict__ st, int p, unsigned long long rank0,
-                                          unsigned nblocks) {
+                                          unsigned nblocks, const unsigned* __restrict__ prev_hist = nullptr) {
     using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
@@ -89,7 +89,7 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
     s.mask = 0ull;
     s.rank = rank0;
     if (p > 0) {
-        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above);
+        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above, prev_hist);
         if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
     }
     for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
@@ -165,7 +165,8 @@ __global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict
 // patterns, i.e. a vector of |x|) when they hold the wanted rank and all fit their buffer, the whole
 // vector(s) otherwise.  Every pass of a selection reads the same count and decides alike, so the
 // host launches the passes without knowing which way they go.  The grid is sized for the whole
-// vector; over the candidates only the blocks they need stay.
+// vector; over the candidates only the blocks they need stay, and pass 0 has nothing to do: the
+// kernel that collected them left their top-digit counts behind the last pass's histogram.
 template <typename T, bool HAS_ADD, int VEC>
 __global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                                     long long m,
@@ -173,13 +174,15 @@ __global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __r
                                                                     unsigned cap, const unsigned* __restrict__ cand_count,
                                                                     SelectState* __restrict__ st, int p,
                                                                     unsigned long long rank0) {
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     const unsigned count = *cand_count;
     if ((unsigned long long)count > rank0 && count <= cap) {
+        if (p == 0) return;
         constexpr unsigned kPerBlock = (unsigned)kBlock * VEC * 8u;
         unsigned need = (count + kPerBlock - 1u) / kPerBlock;
         if (need > gridDim.x) need = gridDim.x;
         hist_pass<T, 0, false, VEC>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
-                                    st, p, rank0, need);
+                                    st, p, rank0, need, p == 1 ? st->pass_hist[kPasses] : nullptr);
     } else {
         hist_pass<T, 0, HAS_ADD, VEC>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
     }
@@ -619,11 +622,16 @@ template <typename T, bool HAS_ADD, int VEC>
 __global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                                 long long m, const T* __restrict__ d_bound,
                                                                 typename Elem<T>::key_t* __restrict__ cand, unsigned cap,
-                                                                unsigned* __restrict__ cand_count, int reverse) {
+                                                                unsigned* __restrict__ cand_count, int reverse,
+                                                                unsigned* __restrict__ top_hist) {
     using key_t = typename Elem<T>::key_t;
     constexpr int kPerIter = 64 * VEC * kCollectUnroll;  // keys a wavefront looks at per iteration
     constexpr int kSegKeys = 2 * kPerIter;
+    constexpr int shift0 = Elem<T>::key_bits - kRadixBits;
     __shared__ key_t seg[kBlock / 64][kSegKeys];
+    __shared__ unsigned lds_hist[kRadixBins];  // top digits of the block's candidates
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const key_t bound = key_of(*d_bound);
     key_t* my = seg[wave];
@@ -650,7 +658,10 @@ __global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restr
         }
         unsigned at = held + incl - cnt;
         for (int q = 0; q < nkeys; ++q)
-            if ((mask >> q) & 1u) my[at++] = kk[q];
+            if ((mask >> q) & 1u) {
+                my[at++] = kk[q];
+                atomicAdd(&lds_hist[(unsigned)(kk[q] >> shift0)], 1u);
+            }
         held += __shfl(incl, 63, 64);
     };
 
@@ -727,6 +738,11 @@ __global__ __launch_bounds__(kBlock) void select_collect_kernel(const T* __restr
     for (int w = 0; w < wave; ++w) base += s_held[w];
     for (unsigned i = lane; i < held; i += 64)
         if (base + i < cap) cand[base + i] = my[i];
+    // the candidates are the largest keys: they share a few top digits, so this is a few atomics per block
+    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+        const unsigned c = lds_hist[b];
+        if (c) atomicAdd(&top_hist[b], c);
+    }
 }
 
 template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v; }
@@ -886,10 +902,11 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     key_t* cand = static_cast<key_t*>(h->cand);
     if (add_vec)
         hipLaunchKernelGGL((select_collect_kernel<T, true, kVec>), dim3(kCollectBlocks), dim3(kBlock), 0, h->stream, vec, add_vec,
-                           (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse);
+                           (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse, h->sel->pass_hist[kPasses]);
     else
         hipLaunchKernelGGL((select_collect_kernel<T, false, kVec>), dim3(kCollectBlocks), dim3(kBlock), 0, h->stream, vec,
-                           add_vec, (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse);
+                           add_vec, (long long)m, d_bound, cand, (unsigned)cap, d_count, reverse,
+                           h->sel->pass_hist[kPasses]);
     // 3. the passes, over whichever the count allows
     const long long per_block = (long long)kBlock * kVec * 8;
     long long blocks = ((long long)m + per_block - 1) / per_block;
