@@ -364,6 +364,60 @@ def test_optimizer_over_ranks_adds_up_to_the_closed_form(schedule):
         assert all(held_back[r] > 0 for r in range(R))
 
 
+def test_exact_whole_vector_step_can_be_captured_in_a_hip_graph(oracle):
+    """The exact whole-vector threshold on a long vector (sampled bound, candidate pass, radix passes
+    that read the candidate count on the device) and the compress behind it wait for nothing, so they
+    can be captured: two steps replayed three times, with eager work and synchronisations between the
+    replays, give the eager result every time, and the eager result is the checker's."""
+    from comprex_amd.device import Handle, message_capacity
+    rng = np.random.default_rng(43)
+    n = 9_000_001
+    g_h = rng.laplace(size=n).astype(np.float32)
+    g = torch.from_numpy(g_h).cuda()
+    rests = torch.zeros(n, device="cuda")
+    msg = torch.zeros(message_capacity(n, torch.float32), dtype=torch.uint8, device="cuda")
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        h = Handle()
+        h.reserve(n, torch.float32, Handle.RESERVE_ALL)
+
+        def step():
+            h.topk_threshold(rests, g, np.float32(0.002), 1 << 30, to_host=False)
+            h.compress(msg, g, rests, sync=False)
+
+        for _ in range(2):
+            step()
+        side.synchronize()
+        rests.zero_()
+        step(), step()
+        side.synchronize()
+        want_rests = rests.clone()
+        want_msg = msg[: 8 + 8 * int(msg[4:8].view(torch.int32).item())].clone()
+        # the checker on the same two steps
+        r_h = np.zeros(n, np.float32)
+        for _ in range(2):
+            thr = oracle.topk_prepare_with(r_h, g_h, np.float32(0.002), 1 << 30, 10.0)
+            ref_msg = oracle.ip_compress(g_h, r_h, np.float32(thr))
+        assert want_msg.cpu().numpy().tobytes() == ref_msg.tobytes()
+        assert want_rests.cpu().numpy().tobytes() == r_h.tobytes()
+        rests.zero_()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(), step()
+        side.synchronize()
+        for _ in range(3):
+            rests.zero_()
+            msg.zero_()
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            k = int(msg[4:8].view(torch.int32).item())
+            assert torch.equal(rests, want_rests)
+            assert torch.equal(msg[: 8 + 8 * k], want_msg)
+        h.synchronize()
+        h.close()
+
+
 def test_sampled_step_can_be_captured_in_a_hip_graph():
     """threshold (left on the device) + compress enqueue kernels only, so a caller may capture them.
     Two steps (one in each walking direction) are captured and replayed three times, with eager
