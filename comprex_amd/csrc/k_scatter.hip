@@ -656,7 +656,8 @@ __global__ __launch_bounds__((MergeCfg<T, ACCUM>::block)) void merge_kernel(T* _
                     vec_t vv;
 #pragma unroll
                     for (int c = 0; c < VEC; ++c) vv[c] = v.x[c];
-                    // (nontemporal: the vector is written once; plain stores measured the same)
+                    // (nontemporal: the vector is written once.  Plain stores: 78 against 52 us from zeros and 100 against
+                    // 95 us adding, 8 messages into 64 Mi fp32 elements; what reads the vector next gains nothing)
                     __builtin_nontemporal_store(vv, reinterpret_cast<vec_t*>(out + base + e));
                 } else if (draining) {
 #pragma unroll
