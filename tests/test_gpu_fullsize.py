@@ -56,7 +56,11 @@ def _error_feedback(dev, oracle, cfg, grad_fn, iters, gold_rows, oracle_live=Tru
     for it in range(iters):
         g_h = grad_fn(it)
         g = torch.from_numpy(g_h).cuda()
-        if fused_route is None:
+        if fused_route == "step":
+            # threshold and compress enqueued by ONE call (what ComprEx::writeRemote uses)
+            nbytes = dev.write_step(buf, g, rests, topk, ds, d_thr=thr_out)
+            thr = float(thr_out.item())
+        elif fused_route is None:
             thr = dev.topk_threshold(rests, g, topk, ds)
             nbytes = dev.compress(buf, g, rests)  # threshold from the handle's device slot
         else:
@@ -96,6 +100,15 @@ def test_c1_and_c3_threshold_and_compress_as_one_call(dev, oracle):
     # C1 is too small for the single pass (route 0), C3 takes it (route 1); same recorded outputs
     assert _error_feedback(dev, oracle, W.C1, W.c1_gradient, 3, GOLD["C1"], fused_route=0) == 3
     assert _error_feedback(dev, oracle, W.C3, W.c3_gradient, 3, GOLD["C3"], fused_route=1) == 3
+
+
+def test_c1_c2_c3_write_step_one_call(dev, oracle):
+    """cx_ip_write_step on the reference's configurations: chained radix passes (C1), the two-launch
+    select (C2), the single pass over both vectors (C3); the recorded reference outputs and the
+    live checker."""
+    assert _error_feedback(dev, oracle, W.C1, W.c1_gradient, W.C1["iters"], GOLD["C1"], fused_route="step") == W.C1["iters"]
+    assert _error_feedback(dev, oracle, W.C2, W.c2_gradient, W.C2["iters"], GOLD["C2"], fused_route="step") == W.C2["iters"]
+    assert _error_feedback(dev, oracle, W.C3, W.c3_gradient, 4, GOLD["C3"], fused_route="step") == 4
 
 
 def test_c3_resnet50_top0p1pct(dev, oracle):

@@ -98,6 +98,39 @@ def test_reserve_takes_the_scratch_up_front(oracle):
         h.close()
 
 
+def test_write_step_equals_prepare_with_then_compress(dev, oracle):
+    """cx_ip_write_step = ThresholdTopK(topK, default_subsamples, factor).prepare_with(residual, gradient)
+    followed by compress_add_update, in the reference's three sampling modes (strided sample, whole
+    vector because the sample would cover it, and caller-given positions), three element types, over
+    residual-carrying steps: threshold, message and residual equal the checker's."""
+    from comprex_amd.device import message_capacity
+    rng = np.random.default_rng(77)
+    for dtype in DTYPES:
+        tdt = NP2T[dtype]
+        for n, topk, ds, indexed in ((100_003, 0.01, 1000, False), (100_003, 0.05, 1 << 20, False),
+                                     (1_500_001, 0.002, 1 << 22, False), (300_000, 0.02, 1000, True),
+                                     (5, 0.5, 1000, False), (1, 0.5, 1000, False)):
+            say("write_step", dtype.__name__, n, topk, ds, indexed)
+            r_h = np.zeros(n, dtype)
+            r = torch.zeros(n, dtype=tdt, device="cuda")
+            buf = torch.zeros(message_capacity(n, tdt), dtype=torch.uint8, device="cuda")
+            thr_out = torch.zeros(1, dtype=tdt, device="cuda")
+            idx_h = rng.integers(0, n, 20_000).astype(np.int32) if indexed else None
+            idx = _gpu(idx_h) if indexed else None
+            for step in range(3):
+                g_h = (rng.standard_normal(n) * (1000 if dtype == np.int32 else 1)).astype(dtype)
+                g = _gpu(g_h)
+                nbytes = dev.write_step(buf, g, r, np.float32(topk), ds, 10.0, idx=idx, d_thr=thr_out)
+                if indexed:
+                    want_thr = oracle.topk_prepare_indexed(r_h, g_h, idx_h, np.float32(topk))
+                else:
+                    want_thr = oracle.topk_prepare_with(r_h, g_h, np.float32(topk), ds, 10.0)
+                want = oracle.ip_compress(g_h, r_h, dtype(want_thr))
+                assert thr_out.cpu().numpy()[0] == dtype(want_thr), (dtype.__name__, n, step)
+                assert nbytes == want.size and buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
+                assert r.cpu().numpy().tobytes() == r_h.tobytes()
+
+
 # --------------------------------------------------------------------------- K2
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("mode", ["fused", "update", "data"])
