@@ -478,6 +478,24 @@ def main():
                                 "frac": acc_bytes / (acc_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}
         log("reduce ordered, added into the vector %.3f ms (%.0f GB/s of 8n+16Rk, %.1f%% of peak)"
             % (acc_ms, reduce["accumulate"]["GBps"], 100 * reduce["accumulate"]["frac"]))
+        # the same shape in fp64: half as many elements (the same 256 MB vector), 1 %-dense messages of
+        # 12-byte pairs; per pair 12 B of message + 8 B read + 8 B write, the vector read and written
+        n64, k64 = c5n // 2, c5k // 2
+        msgs64 = [torch.from_numpy(mm).cuda() for mm in W.c5_messages(n=n64, k=k64, shared=k64 // 2, dtype=np.float64)]
+        dense64 = torch.zeros(n64, dtype=torch.float64, device="cuda")
+        f64 = {}
+        for acc, key, nbytes in ((False, "from_zeros", 8 * n64 + 28 * len(msgs64) * k64),
+                                 (True, "accumulate", 16 * n64 + 28 * len(msgs64) * k64)):
+            for _ in range(2):
+                h.reduce(dense64, msgs64, accumulate=acc, mode=0)
+            ms64 = event_ms(torch, lambda: h.reduce(dense64, msgs64, accumulate=acc, mode=0), reps)
+            f64[key] = {"algorithmic_bytes": nbytes, "ms": ms64, "GBps": nbytes / (ms64 * 1e-3) / 1e9,
+                        "frac": nbytes / (ms64 * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+        reduce["f64"] = dict(f64, n=n64, k_per_rank=k64)
+        log("reduce ordered, fp64 (%d elements): from zeros %.3f ms (%.1f%% of peak of 8n+28Rk), added into the vector "
+            "%.3f ms (%.1f%% of peak of 16n+28Rk)" % (n64, f64["from_zeros"]["ms"], 100 * f64["from_zeros"]["frac"],
+                                                       f64["accumulate"]["ms"], 100 * f64["accumulate"]["frac"]))
+        del msgs64, dense64
         # The chief's apply as the reference runs it (src/allreduce.tpp:183-205): readRemote_add per
         # worker into its own vector (here ONE rank-ordered accumulate), then the broadcast leg's
         # writeRemote(data): residual += reduced vector, exact top-k 1 %, compact, zero
