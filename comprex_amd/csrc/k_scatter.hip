@@ -357,7 +357,8 @@ constexpr int kPrefillAhead = 2;
 //   adding (4 more loader wavefronts, 2 more buffers) and 8-byte elements (12-byte pairs): two
 //     messages per wavefront; rings of 4 x 128 pairs for 4-byte elements adding (144 KB) and for
 //     8-byte elements from zeros (128 KB), 4 x 64 pairs for 8-byte elements adding (136 KB; with
-//     8 KB tiles instead: 118 us against 97 us).
+//     8 KB tiles instead: 118 us against 97 us).  8-byte elements from zeros with one message per
+//     wavefront need smaller tiles to fit (9 x 12 KB + 24 KB): 87 us against 68 us.
 //   Writer wavefronts: 4 when writing from zeros (52 us against 59 us with 8, 69 us with 2: the
 //     stores of more wavefronts queue up behind each other), 8 when adding (no difference there).
 template <typename T, bool ACCUM> struct MergeCfg {
