@@ -383,6 +383,52 @@ def main():
         log("plain streaming on this GPU: copy %.0f GB/s, in-place add %.0f GB/s"
             % (extra["device_copy_GBps"], extra["inplace_add_GBps"]))
 
+        # The same step with the vector cut into S contiguous segments, each with a handle and a stream
+        # of its own (what Comprex_RingAllreduce's per-segment ComprEx objects amount to on one GPU,
+        # src/allreduce.tpp:372-416): the segments' latency-bound small kernels run beside the other
+        # segments' streaming kernels.  The cached tail of the residual is shared out among the segments.
+        seg_out = {}
+        for S in (2, 4):
+            seg = (n // S) & ~3
+            streams = [torch.cuda.Stream() for _ in range(S)]
+            hs, seg_msgs, seg_idx = [], [], []
+            for q in range(S):
+                with torch.cuda.stream(streams[q]):
+                    hs.append(Handle())
+                hs[q].set_option("stage_cached_tail_mb", 192 // S)
+                seg_msgs.append(torch.zeros(message_capacity(seg, torch.float32) // 8, dtype=torch.uint8, device="cuda"))
+                pos = idx_h[(idx_h >= q * seg) & (idx_h < (q + 1) * seg)] - q * seg
+                seg_idx.append(torch.from_numpy(pos.astype(np.int32)).cuda())
+
+            def seg_steps():
+                for q in range(S):
+                    with torch.cuda.stream(streams[q]):
+                        gq, rq = g[q * seg:(q + 1) * seg], rests[q * seg:(q + 1) * seg]
+                        hs[q].topk_threshold_indexed(rq, gq, seg_idx[q], topk, to_host=False)
+                        hs[q].compress(seg_msgs[q], gq, rq, sync=False)
+
+            torch.cuda.synchronize()
+            for _ in range(5):
+                seg_steps()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(30):
+                seg_steps()
+            torch.cuda.synchronize()
+            seg_ms = (time.perf_counter() - t0) / 30 * 1e3
+            ks = sum(int(mq[4:8].view(torch.int32).item()) for mq in seg_msgs)
+            seg_bytes = 12 * S * seg + 8 * ks + 8 * S + 8 * sum(int(t.numel()) for t in seg_idx)
+            seg_out[str(S)] = {"ms": seg_ms, "GBps": seg_bytes / (seg_ms * 1e-3) / 1e9,
+                               "frac": seg_bytes / (seg_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "k": ks,
+                               "cached_tail_mb_each": 192 // S}
+            for hq in hs:
+                hq.synchronize()
+                hq.close()
+            del seg_msgs, seg_idx
+        extra["segments_on_own_streams"] = seg_out
+        log("the step as 2 / 4 segments on streams of their own: %.3f / %.3f ms (one stream: %.3f ms)"
+            % (seg_out["2"]["ms"], seg_out["4"]["ms"], ms_per_step))
+
         # exact top-k (radix select over all n) + compress, same vector
         rests.zero_()
         ds = W.C4["default_subsamples_exact"] if n == W.C4["n"] else 1 << 30
