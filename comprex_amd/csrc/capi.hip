@@ -284,10 +284,14 @@ int cx_create(cx_handle* out, void* hip_stream) {
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&h->d_status), 256);
     if (e == hipSuccess) e = hipMalloc(&h->d_thr, 256);
     if (e == hipSuccess) e = hipHostMalloc(reinterpret_cast<void**>(&h->h_pinned), 64, hipHostMallocDefault);
-    if (e == hipSuccess) e = hipMemset(h->redo_flag, 0, 256);
-    if (e == hipSuccess) e = hipMemset(h->sel, 0, sizeof(SelectState));
-    if (e == hipSuccess) e = hipMemset(h->d_status, 0, 256);
-    if (e == hipSuccess) e = hipMemset(h->d_thr, 0, 256);
+    // cleared ON THE HANDLE'S STREAM and waited for: a plain hipMemset runs on the null stream, with
+    // which a non-blocking stream is not ordered, so a first kernel could see (or a late memset wipe)
+    // the state of whoever held this memory before
+    if (e == hipSuccess) e = hipMemsetAsync(h->redo_flag, 0, 256, h->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(h->sel, 0, sizeof(SelectState), h->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(h->d_status, 0, 256, h->stream);
+    if (e == hipSuccess) e = hipMemsetAsync(h->d_thr, 0, 256, h->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(h->stream);
     if (e != hipSuccess) {
         cx_destroy(h);
         return fail(CX_ERR_HIP, "cx_create: %s", hipGetErrorString(e));

@@ -460,3 +460,47 @@ def test_sampled_step_can_be_captured_in_a_hip_graph():
             assert torch.equal(rests, want_rests)
             assert torch.equal(msg[: 8 + 8 * k], want_msg)
         h.synchronize()
+
+
+def test_handle_on_a_stream_of_its_own_starts_from_clean_state(oracle):
+    """A handle created on a non-blocking stream clears its status words, select state and flags on
+    THAT stream before cx_create returns (the null stream, where a plain memset runs, is not ordered
+    with such a stream): device memory that held other bytes just before must not show through as a
+    device-side error or a wrong threshold."""
+    import ctypes as C
+    from comprex_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(3)
+    n = 20_000
+    v_h = rng.standard_normal(n).astype(np.float32)
+    v = torch.from_numpy(v_h).cuda()
+    want = oracle.topk_prepare(v_h, np.float32(0.05), 1 << 20, 10.0)
+    junk_h = np.full(1 << 16, 0x5a5a5a5a, np.uint32)
+    torch.cuda.synchronize()
+    for _ in range(25):
+        # bytes other than zero in memory of the sizes a handle allocates, then free it again
+        held = []
+        for size in (256, 256, 256, 1 << 16, 1 << 17):
+            p = C.c_void_p()
+            _lib.check(L.cx_device_alloc(C.byref(p), size))
+            held.append((p, size))
+        tmp = C.c_void_p()
+        _lib.check(L.cx_create(C.byref(tmp), None))
+        for p, size in held:
+            _lib.check(L.cx_copy(tmp, p, C.c_void_p(junk_h.ctypes.data), size))
+        _lib.check(L.cx_synchronize(tmp))
+        for p, _size in held:
+            _lib.check(L.cx_device_free(p))
+        L.cx_destroy(tmp)
+        stream, h = C.c_void_p(), C.c_void_p()
+        _lib.check(L.cx_stream_create(C.byref(stream)))
+        _lib.check(L.cx_create(C.byref(h), stream))
+        try:
+            _lib.check(L.cx_synchronize(h))  # a status word that is not zero would be reported here
+            thr = C.c_float(0)
+            _lib.check(L.cx_topk_threshold(h, _lib.CX_F32, C.c_void_p(v.data_ptr()), None, n, 0, C.c_float(0.05),
+                                           1 << 20, C.c_float(10.0), None, C.byref(thr)))
+            assert thr.value == want
+        finally:
+            L.cx_destroy(h)
+            L.cx_stream_destroy(stream)
