@@ -978,7 +978,9 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
     if (rc != CX_OK) return rc;
     // 3. threshold among the candidates
     // (chained passes: the pick after each pass is redone by every block of the next kernel, the
-    // last one by the filter, which also writes the threshold and clears the histograms)
+    // last one by the filter, which also writes the threshold and clears the histograms).  Blocks per
+    // pass, measured as the whole call on 100 M fp32 elements at 1 % / on 25.6 M at 0.1 %: 64 blocks
+    // 0.340 ms / 120 us, 128 0.304 / 117, 256 0.297 / 121, 512 0.304 / 123, 1024 0.318 / 124.
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     for (int p = 0; p < kPasses; ++p)
         hipLaunchKernelGGL(select_hist_pairs_kernel<T>, dim3(256), dim3(kBlock), 0, h->stream, cand_words, (unsigned)cap,
