@@ -41,11 +41,11 @@ namespace {
 constexpr int kBlock = 256;
 constexpr int kWavesPerBlock = kBlock / 64;
 constexpr unsigned kDeferred = 0x80000000u;
-// threads of a gather block and pairs a lane moves per round.  Measured, whole step as above: 128 / 256 /
-// 512 threads and 2 / 4 / 8 pairs all give 0.208 ms (0.222-0.223 ms after the gradient was rewritten); on
-// 61 706 elements at 10 % the threshold + compress take 50 / 42 / 41 us with 128 / 256 / 512 threads and
-// 44 / 42 / 42 us with 2 / 4 / 8 pairs.
-constexpr int kGatherBlock = 256;
+// threads of a gather block and pairs a lane moves per round.  Measured, whole step on 100 M fp32
+// elements at 1 % / threshold + compress on 61 706 elements at 10 % (one gather block moves all 6 170
+// pairs there): 256 threads x 4 pairs 0.208 ms / 40.5 us, 256 x 8 0.209 / 40.2, 512 x 4 0.208 / 38.7,
+// 512 x 8 0.212 / 37.9, 128 x 4 0.208 / 50 (measured with deferred tiles in the short vector).
+constexpr int kGatherBlock = 512;
 constexpr int kGatherUnroll = 4;
 constexpr int kGatherTiles = 64;                // tiles a gather block owns: one lane per tile in its scan
 static_assert(kGatherTiles % (kWavesPerBlock * 8) == 0, "a gather block's streaming blocks fill whole 16-byte loads of 16-bit sums");
@@ -131,9 +131,9 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
                                              unsigned* __restrict__ counts,
                                              unsigned* __restrict__ redo_flag, unsigned epoch,
                                              unsigned* __restrict__ out_pairs, long long direct_pos,
-                                             long long cap_pairs, DeviceStatus* status, bool nt_update = false) {
+                                             long long cap_pairs, DeviceStatus* status, bool nt_update = false,
+                                             unsigned slot_pairs = 0u) {
     constexpr int kTile = 64 * VEC * ITEMS;
-    constexpr int kCap = kTile / 8;
     constexpr int PW = Elem<T>::pair_words;
     const long long base = (long long)tile * kTile;
     const bool full = base + kTile <= n;
@@ -203,7 +203,7 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
         dst = out_pairs + direct_pos * PW;
         dst_limit = cap_pairs - direct_pos;
     } else {
-        if (total > (unsigned)kCap) {
+        if (total > slot_pairs) {
             if (lane == 0) {
                 counts[tile] = total | kDeferred;
                 *redo_flag = epoch;
@@ -211,8 +211,8 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
             return total;  // no side effects: the redo pass starts from untouched inputs
         }
         if (lane == 0) counts[tile] = total;
-        dst = staging + (long long)tile * (kCap * PW);
-        dst_limit = kCap;
+        dst = staging + (long long)tile * (long long)(slot_pairs * (unsigned)PW);
+        dst_limit = slot_pairs;
     }
 
     bool overflow = false;
@@ -257,7 +257,8 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
                                                        unsigned* __restrict__ staging, unsigned* __restrict__ counts,
                                                        unsigned* __restrict__ block_sums,
                                                        unsigned* __restrict__ redo_flag, unsigned epoch,
-                                                       unsigned ntiles, int reverse, unsigned cached_from) {
+                                                       unsigned ntiles, int reverse, unsigned cached_from,
+                                                       unsigned slot_pairs) {
     // survivors of this block's tiles, summed in LDS; the wavefront that finishes last stores
     // the sum, which spares the gather kernel a scan over every tile count
     __shared__ unsigned s_sum, s_done;
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
     const bool nt_update = __builtin_amdgcn_readfirstlane((int)(walk_rank < cached_from)) != 0;
     const unsigned total = process_tile<T, MODE, VEC, ITEMS, false>(data, update, n, thr, tile, threadIdx.x & 63,
                                                                     staging, counts, redo_flag, epoch, nullptr, 0, 0,
-                                                                    nullptr, nt_update);
+                                                                    nullptr, nt_update, slot_pairs);
     if ((threadIdx.x & 63) == 0) {
         const unsigned tiles_here = ntiles - block * kWavesPerBlock < (unsigned)kWavesPerBlock
                                         ? ntiles - block * kWavesPerBlock
@@ -323,9 +324,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     const T* __restrict__ data, T* __restrict__ update, long long n, const T* __restrict__ thr_ptr, T thr_val,
     const unsigned* __restrict__ counts, const unsigned* __restrict__ block_sums, unsigned* __restrict__ offsets,
     const unsigned* __restrict__ staging, unsigned ntiles, unsigned* __restrict__ msg_words, long long cap_pairs,
-    int* __restrict__ size_prefix, int inline_redo, DeviceStatus* status) {
+    int* __restrict__ size_prefix, int inline_redo, DeviceStatus* status, unsigned slot_pairs) {
     constexpr int PW = Elem<T>::pair_words;
-    constexpr int kSlotPairs = 64 * VEC * ITEMS / 8;
     constexpr int kWaves = kGatherBlock / 64;
     // pairs a lane moves per round: searches and loads of one round are independent
     constexpr int kCopyUnroll = kGatherUnroll;
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
             for (int step = 32; step > 0; step >>= 1)
                 lo += (s_off[lo + step > 63 ? 63 : lo + step] <= p && lo + step <= 63) ? step : 0;
             if ((deferred >> lo) & 1ull) live[q] = false;  // not staged
-            src_idx[q] = (first + lo) * (unsigned)kSlotPairs + (p - s_off[lo]);
+            src_idx[q] = (first + lo) * slot_pairs + (p - s_off[lo]);
         }
 #pragma unroll
         for (int q = 0; q < kCopyUnroll; ++q)
@@ -474,6 +474,8 @@ struct Scratch {
 // contents of an earlier call are harmless; two calls that overlap in time on one GPU would race.
 constexpr long long kNoAllocMaxN = 1ll << 24;
 constexpr size_t kStaticStagingWords = (size_t)kNoAllocMaxN * 3 / 8 + 1024;
+// vectors up to this length get staging slots that hold a whole tile (32 to 48 MB of staging at most)
+constexpr long long kWholeSlotMaxN = 1ll << 22;
 constexpr size_t kStaticTiles = (size_t)kNoAllocMaxN / 256 + 64;
 constexpr size_t kStaticSumsWords = kStaticTiles / 4 + 64;
 constexpr size_t kStaticWords = kStaticStagingWords + 2 * kStaticTiles + kStaticSumsWords;
@@ -514,22 +516,32 @@ template <typename T> void scratch_need(long long n, size_t* ntiles, size_t* sta
     constexpr int PW = Elem<T>::pair_words;
     constexpr long long kSmallestTile = 64ll * kVec * 2, kLargestTile = 64ll * kVec * 8;
     *ntiles = (size_t)((n + kSmallestTile - 1) / kSmallestTile);
-    *staging_words = (size_t)((n + kLargestTile - 1) / kLargestTile) * (size_t)(kLargestTile / 8) * PW;
+    const size_t slot = n <= kWholeSlotMaxN ? (size_t)kLargestTile : (size_t)(kLargestTile / 8);  // as launch_all chooses
+    *staging_words = (size_t)((n + kLargestTile - 1) / kLargestTile) * slot * PW;
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
 int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T thr_val, unsigned* msg_words,
                long long cap_pairs, int* size_prefix, DeviceStatus* status, bool no_alloc) {
     constexpr int kTile = 64 * VEC * ITEMS;
-    constexpr int kCap = kTile / 8;
     constexpr int PW = Elem<T>::pair_words;
     const unsigned ntiles = (unsigned)(((long long)n + kTile - 1) / kTile);
+    // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
+    // the second pass then gets the whole GPU instead of the gather kernel's few blocks
+    const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
+    // Pairs a tile's staging slot holds.  An eighth of the tile keeps the staging area small on long
+    // vectors (a tile with more survivors is deferred and processed again in the gather kernel, one
+    // wavefront per tile).  Short vectors get whole-tile slots: nothing is ever deferred there, and
+    // their gather kernel has too few blocks to hide such repeats (61 706 elements at 10 %: 3 to 5
+    // deferred tiles made the gather kernel 11 us long instead of 5).
+    const bool whole_slots = !no_alloc && MODE != 3 && !dense_hint && (long long)n <= kWholeSlotMaxN;
+    const unsigned slot_pairs = whole_slots ? (unsigned)kTile : (unsigned)kTile / 8u;
     Scratch sc;
     if (no_alloc) {
         // the per-GPU static array, cut into the four arrays; never grows
         unsigned* base = h->static_scratch;
         if (!base) return fail(CX_ERR_INTERNAL, "compress: the static scratch array was not located on this device");
-        if ((size_t)ntiles * kCap * PW > kStaticStagingWords || (size_t)ntiles > kStaticTiles ||
+        if ((size_t)ntiles * slot_pairs * PW > kStaticStagingWords || (size_t)ntiles > kStaticTiles ||
             (size_t)(ntiles + kWavesPerBlock - 1) / kWavesPerBlock > kStaticSumsWords)
             return fail(CX_ERR_INVALID, "compress: %d elements exceed the static scratch array", n);
         sc.staging = base;
@@ -537,7 +549,7 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
         sc.offsets = sc.counts + kStaticTiles;
         sc.block_sums = sc.offsets + kStaticTiles;
     } else {
-        int rc = ensure_scratch(h, ntiles, (size_t)ntiles * kCap * PW);
+        int rc = ensure_scratch(h, ntiles, (size_t)ntiles * slot_pairs * PW);
         if (rc != CX_OK) return rc;
         sc.staging = h->staging;
         sc.counts = h->tile_counts;
@@ -565,16 +577,13 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
     }
     hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
                        (long long)n, thr_ptr, thr_val, sc.staging, sc.counts, sc.block_sums, redo_flag, h->epoch, ntiles,
-                       reverse, cached_from);
+                       reverse, cached_from, slot_pairs);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
-    // a threshold known to select (nearly) everything, as flushRests passes, defers every tile:
-    // give the second pass the whole GPU instead of the gather kernel's few blocks
-    const int dense_hint = (thr_ptr == nullptr && !(thr_val > (T)0)) ? 1 : 0;
     const unsigned gather_blocks = (ntiles + kGatherTiles - 1) / kGatherTiles;
     hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
                        update, (long long)n, thr_ptr, thr_val, sc.counts, sc.block_sums,
                        sc.offsets, sc.staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
-                       status);
+                       status, slot_pairs);
     if (dense_hint) {
         const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
         hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
