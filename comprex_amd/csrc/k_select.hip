@@ -813,25 +813,38 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     using key_t = typename Elem<T>::key_t;
 
+    // short list of the two-launch select: see below
+    int short_k = 0;
+    const unsigned short_cap = (unsigned)kShortGlobalKeys;
     if (m <= kSmallSelect) {
+        const int blocks = (m + kFirstBlock - 1) / kFirstBlock;
+        const double share = (double)(rank + 1) / (double)blocks;
+        short_k = (int)(share + 8.0 * std::sqrt(share) + 8.0);
+        if (!h->select_short_list || m < 8192 || short_k > kFirstBlock / 8 ||
+            (double)blocks * (short_k + 16.0) > (double)short_cap)
+            short_k = 0;
+    }
+    // Two launches or chained passes?  Measured on N(0,1) keys, whole vector (+ second vector), threshold
+    // alone, top 1 % / 3 % / 10 % / 30 %: the chained passes take 20.2 to 21.1 us for any count up to 2^18
+    // and any fraction; the two launches 11.8 / 14.5 / 14.0 / 14.9 us on 40 000 keys, 12.4 / 15.5 / 16.9 /
+    // 18.3 on 61 706, 13.6 / 18.0 / 22.2 / 24.0 on 100 000, 15.6 / 21.9 / 28.2 / 31.1 on 150 000, 17.5 /
+    // 25.5 / 34.7 / 38.6 on 200 000, 19.9 / 49.5 / 40.9 / 38.8 on 262 144: their one-block second launch
+    // grows with what the short list leaves it.  Sampled keys (two dependent gathers per key and pass) and
+    // 8-byte keys (six passes) stay with the two launches.
+    const bool two_launches = m <= kSmallSelect && (sample_mode != kSampleFull || kPasses > 3 || zero_word ||
+                                                     m <= (1 << 16) || (short_k > 0 && rank <= 3000ull));
+    if (two_launches) {
         int rc_keys = ensure_select_keys(h);
         if (rc_keys != CX_OK) return rc_keys;
         key_t* keys = static_cast<key_t*>(h->sel_keys);
         key_t* short_keys = reinterpret_cast<key_t*>(static_cast<char*>(h->sel_keys) + h->sel_keys_bytes);
-        const int per_block = kFirstBlock;
-        const int blocks = (m + per_block - 1) / per_block;
+        const int blocks = (m + kFirstBlock - 1) / kFirstBlock;
         // short list: worth it when the wanted rank is near the top, so that a block's share of the
         // keys above it (plus 8 sigma) is a small part of the block, and the shares fit the list.
         // Measured, threshold alone, list on / off: 200 000 N(0,1) keys, top 1 % 17.9 / 27.6 us, 3 %
         // 25.4 / 34.3 us, 10 % 49.1 / 34.9 us; 61 706 such keys 12.4 / 14.7, 15.7 / 16.9, 19.3 / 16.9 us;
         // 61 706 keys in segments of very different scale (the list can never decide there) 18.1 / 13.5,
         // 19.4 / 14.4, 22.4 / 16.6 us.  Hence an eighth of the block at most (top 5 % or so).
-        const unsigned short_cap = (unsigned)kShortGlobalKeys;
-        const double share = (double)(rank + 1) / (double)blocks;
-        int short_k = (int)(share + 8.0 * std::sqrt(share) + 8.0);
-        if (!h->select_short_list || m < 8192 || short_k > per_block / 8 ||
-            (double)blocks * (short_k + 16.0) > (double)short_cap)
-            short_k = 0;
 #define CX_FIRST(SM, HA)                                                                                             \
     hipLaunchKernelGGL((select_first_kernel<T, SM, HA>), dim3(blocks), dim3(kFirstBlock), 0, h->stream, vec, add_vec, \
                        d_idx, m, n, stepsize, keys, h->sel, short_k, short_keys, short_cap)
