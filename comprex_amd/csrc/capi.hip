@@ -418,7 +418,7 @@ int cx_set_option(cx_handle h, const char* key, int value) {
         if (value < 1 || value > 32) return fail(CX_ERR_INVALID, "reduce_blocks_per_cu must be 1..32");
         h->reduce_blocks_per_cu = value;
     } else if (!strcmp(key, "fused_topk")) {
-        h->fused_topk = value ? 1 : 0;
+        h->fused_topk = value < 0 ? 0 : (value > 2 ? 2 : value);  // 2: from 2^23 elements on, whatever is faster
     } else if (!strcmp(key, "select_short_list")) {
         h->select_short_list = value ? 1 : 0;
 

@@ -125,7 +125,7 @@ struct cx_handle_s {
     int stage_cached_tail_mb = 192;    // residual read cacheably over the last so many MB of a walk (-1: all of it)
     int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound
     int select_short_list = 1;         // 1 = the two-launch select passes a short list of top keys to its second launch
-    int fused_topk = 1;                // 1 = cx_ip_compress_topk may take its single-pass route
+    int fused_topk = 1;                // cx_ip_compress_topk's single-pass route: 0 never, 1 from 20 Mi elements, 2 from 2^23
     int fused_topk_taken = 0;          // how the last cx_ip_compress_topk ran: 0 two calls, 1 single pass, 2 single pass abandoned
     int reduce_variant = 0;            // 0 = rank-ordered, kernel chosen by message count; 1 = per-message scatter;
                                        // 2 = always one block per tile behind a bounds pass; 3 = always the pipelined kernel

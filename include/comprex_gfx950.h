@@ -118,7 +118,8 @@ int cx_synchronize(cx_handle h);
  * "stage_alternate" (1 = every other compress walks the vector from its end, so that it starts on
  * what the previous one left in the memory-side cache), "profile_stage" (see cx_profile_read),
  * "reduce_variant", "select_bracket" (1 = whole-vector thresholds try a one-pass selection first),
- * "fused_topk" (1 = cx_ip_compress_topk may take its single-pass route).  Unknown keys return
+ * "fused_topk" (0 = cx_ip_compress_topk never takes its single-pass route, 1 = where it is the
+ * faster one, from 20 Mi elements on, 2 = from 2^23 elements on).  Unknown keys return
  * CX_ERR_INVALID. */
 int cx_set_option(cx_handle h, const char* key, int value);
 /* Reads an option back; also "fused_topk_taken": how the last cx_ip_compress_topk ran

@@ -60,6 +60,7 @@ def test_reserve_takes_the_scratch_up_front(oracle):
     idx = _gpu(np.sort(rng.integers(0, n, 50_000)).astype(np.int32))
     dense = torch.zeros(n, device="cuda")
     def calls(h, check):
+        h.set_option("fused_topk", 2)   # the single pass from 2^23 elements on (by default only where it is faster)
         thr = h.topk_threshold_indexed(r, g, idx, np.float32(0.01))
         nbytes = h.compress(msg, g, r)
         if check:
@@ -262,7 +263,11 @@ def test_compress_capacity_and_size_errors(dev):
             if route == "flush":
                 dev.compress(tiny, g, r, thr=0.0)
             elif route == "topk":
-                dev.compress_topk(tiny, g, r, np.float32(0.001))
+                dev.set_option("fused_topk", 2)  # the single pass at this length
+                try:
+                    dev.compress_topk(tiny, g, r, np.float32(0.001))
+                finally:
+                    dev.set_option("fused_topk", 1)
             else:
                 dev.rle_compress(tiny, g, r, thr=1.0)
         assert e.value.code == _lib.CX_ERR_CAPACITY, route
@@ -375,7 +380,7 @@ def test_fused_exact_topk_single_pass_and_changes_of_plan(dev, oracle, dtype):
             want_thr = oracle.topk_prepare_with(u, d, t, ds, 10.0)
             uu = u.copy()
             want_msg = oracle.ip_compress(d.copy(), uu, want_thr)
-            for fused in (1, 0):
+            for fused in (2, 0):  # 2: the single pass from 2^23 elements on
                 say("fused exact top-k", dtype.__name__, name, "fused_topk", fused)
                 dev.set_option("fused_topk", fused)
                 gu, gd = _gpu(u), _gpu(d)
@@ -410,8 +415,12 @@ def test_fused_exact_topk_message_buffer_too_small_and_bad_arguments(dev, oracle
     buf = torch.zeros(keep, dtype=torch.uint8, device="cuda")
     gu, gd = _gpu(u), _gpu(d)
     say("fused exact top-k, message buffer too small")
-    with pytest.raises(ComprexError) as e:
-        dev.compress_topk(buf, gd, gu, t)
+    dev.set_option("fused_topk", 2)  # the single pass at this length
+    try:
+        with pytest.raises(ComprexError) as e:
+            dev.compress_topk(buf, gd, gu, t)
+    finally:
+        dev.set_option("fused_topk", 1)
     assert e.value.code == _lib.CX_ERR_CAPACITY
     assert dev.get_option("fused_topk_taken") == 1
     got = buf.cpu().numpy()
