@@ -307,6 +307,20 @@ def test_topk_threshold_matches_oracle(dev, oracle, dtype):
             assert dev.topk_threshold(gv, None, t, ds, sf) == want
 
 
+def test_exact_threshold_on_both_sides_of_the_candidate_pass_limit(dev, oracle):
+    """Whole-vector thresholds just below and at the length from which one candidate pass replaces the
+    three histogram passes (5 Mi elements): the checker's bits on both sides."""
+    rng = np.random.default_rng(29)
+    for n in ((5 << 20) - 1, 5 << 20, (5 << 20) + 3):
+        v = rng.laplace(size=n).astype(np.float32)
+        a = (0.1 * rng.standard_normal(n)).astype(np.float32)
+        gv, ga = _gpu(v), _gpu(a)
+        for topk in (0.0005, 0.02):
+            say("candidate pass limit", n, topk)
+            want = oracle.topk_prepare_with(v, a, np.float32(topk), 1 << 24, 10.0)
+            assert dev.topk_threshold(gv, ga, np.float32(topk), 1 << 24, 10.0) == want
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_exact_threshold_one_pass_bracket_and_fallbacks(dev, oracle, dtype):
     """Whole-vector (exact top-k) thresholds on vectors large enough for the one-pass path
