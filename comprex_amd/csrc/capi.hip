@@ -396,7 +396,7 @@ int cx_synchronize(cx_handle h) {
 int cx_set_option(cx_handle h, const char* key, int value) {
     if (!h || !key) return fail(CX_ERR_INVALID, "null handle or key");
     if (!strcmp(key, "compact_items")) {
-        if (value != 2 && value != 4 && value != 8) return fail(CX_ERR_INVALID, "compact_items must be 2, 4 or 8");
+        if (value != 0 && value != 2 && value != 4 && value != 8) return fail(CX_ERR_INVALID, "compact_items must be 0 (by length), 2, 4 or 8");
         h->compact_items = value;
     } else if (!strcmp(key, "profile_stage")) {
         if (value && !h->profile_events) {

@@ -120,7 +120,7 @@ struct cx_handle_s {
     hipEvent_t* profile_events = nullptr;  // 2 * kProfileRing events, created on first use
 
     // options
-    int compact_items = 4;             // 16-byte loads per lane and tile
+    int compact_items = 0;             // 16-byte loads per lane and tile: 2, 4, 8, or 0 = by the vector's length
     int stage_alternate = 1;           // 1 = every other launch walks the tiles from the end
     int stage_cached_tail_mb = 192;    // residual read cacheably over the last so many MB of a walk (-1: all of it)
     int select_bracket = 1;            // 1 = one-pass whole-vector select with a sampled lower bound

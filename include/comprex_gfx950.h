@@ -114,7 +114,7 @@ int cx_stream_wait_event(void* hip_stream, void* hip_event);
 /* Waits for the handle's stream and returns the first device-side error seen since the
  * last call (CX_OK if none), clearing it. */
 int cx_synchronize(cx_handle h);
-/* Tuning switches: "compact_items" (16-byte loads per lane and tile: 2, 4 or 8),
+/* Tuning switches: "compact_items" (16-byte loads per lane and tile: 2, 4 or 8; 0 = by the vector's length, the default),
  * "stage_alternate" (1 = every other compress walks the vector from its end, so that it starts on
  * what the previous one left in the memory-side cache), "profile_stage" (see cx_profile_read),
  * "reduce_variant", "select_bracket" (1 = whole-vector thresholds try a one-pass selection first),

@@ -181,7 +181,7 @@ def test_compress_variants_agree(dev, oracle, items):
             assert buf[:nbytes].cpu().numpy().tobytes() == want.tobytes()
             assert gu.cpu().numpy().tobytes() == uu.tobytes()
     finally:
-        dev.set_option("compact_items", 4)
+        dev.set_option("compact_items", 0)  # back to the choice by length
 
 
 def test_compress_clustered_survivors(dev, oracle):
