@@ -750,8 +750,14 @@ template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v;
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
 void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long long m, int n, float stepsize, int p,
                  unsigned long long rank0) {
-    const long long per_block = (long long)kBlock * VEC * 8;
-    long long blocks = (m + per_block - 1) / per_block;
+    // Blocks: every block merges its histogram with atomics, few blocks leave memory idle.  Measured,
+    // three passes + pick, with 2 / 4 / 8 / 16 16-byte loads per thread: 150 000 keys 17.0 / 17.9 / 20.6 /
+    // 26.3 us, 2^20 keys 28.7 / 23.9 / 23.6 / 27.9 us, 2^22 keys 73.0 / 49.9 / 38.5 / 37.1 us: about 128
+    // blocks while 2 to 16 loads per thread allow it.
+    const long long fine = (long long)kBlock * VEC * 2, coarse = (long long)kBlock * VEC * 16;
+    const long long at_most = (m + fine - 1) / fine, at_least = (m + coarse - 1) / coarse;
+    long long blocks = at_least > 128 ? at_least : 128;
+    if (blocks > at_most) blocks = at_most;
     if (blocks < 1) blocks = 1;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL((select_hist_kernel<T, SMODE, HAS_ADD, VEC>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
@@ -831,14 +837,15 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
             short_k = 0;
     }
     // Two launches or chained passes?  Measured on N(0,1) keys, whole vector (+ second vector), threshold
-    // alone, top 1 % / 3 % / 10 % / 30 %: the chained passes take 20.2 to 21.1 us for any count up to 2^18
-    // and any fraction; the two launches 11.8 / 14.5 / 14.0 / 14.9 us on 40 000 keys, 12.4 / 15.5 / 16.9 /
-    // 18.3 on 61 706, 13.6 / 18.0 / 22.2 / 24.0 on 100 000, 15.6 / 21.9 / 28.2 / 31.1 on 150 000, 17.5 /
-    // 25.5 / 34.7 / 38.6 on 200 000, 19.9 / 49.5 / 40.9 / 38.8 on 262 144: their one-block second launch
-    // grows with what the short list leaves it.  Sampled keys (two dependent gathers per key and pass) and
-    // 8-byte keys (six passes) stay with the two launches.
+    // alone, top 1 % / 3 % / 10 % / 30 %, two launches against chained passes: 40 000 keys 11.8 / 14.3 /
+    // 14.2 / 14.9 us against 15.6 / 15.5 / 15.4 / 15.7 us, 61 706 keys 12.4 / 15.6 / 16.9 / 18.3 against
+    // 15.9 / 15.8 / 15.6 / 15.8, 100 000 keys 13.6 / 18.1 / 22.2 / 24.0 against 16.0 / 16.3 / 16.1 / 16.4,
+    // 150 000 keys 15.6 / 21.9 / 28.2 / 31.1 against 16.9 / 16.9 / 16.7 / 17.2, 200 000 keys 17.6 / 25.5 /
+    // 34.7 / 38.6 against 17.3 / 17.4 / 17.5 / 18.0, 262 144 keys 20.0 / 49.5 / 40.9 / 38.8 against 18.3 /
+    // 18.5 / 18.6 / 19.4: the one-block second launch grows with what the short list leaves it.  Sampled
+    // keys (two dependent gathers per key and pass) and 8-byte keys (six passes) stay with the two launches.
     const bool two_launches = m <= kSmallSelect && (sample_mode != kSampleFull || kPasses > 3 || zero_word ||
-                                                     m <= (1 << 16) || (short_k > 0 && rank <= 3000ull));
+                                                     m <= 40960 || (short_k > 0 && rank <= 1500ull));
     if (two_launches) {
         int rc_keys = ensure_select_keys(h);
         if (rc_keys != CX_OK) return rc_keys;
