@@ -907,6 +907,9 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     using key_t = typename Elem<T>::key_t;
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     *done = 0;
+    // (sample size, measured on 100 M elements at 1 %: 2^14 / 2^15 / 2^16 / 2^17 samples give 0.153 / 0.155 /
+    // 0.158 / 0.162 ms for this call and 0.306 / 0.301 / 0.297 / 0.297 ms for the single pass below, which uses
+    // the same bound: a smaller sample is cheaper to select from and leaves more candidates)
     constexpr int kSample = 1 << 16;
     const double p = (double)(rank + 1) / (double)m;
     const double expect = p * kSample;
