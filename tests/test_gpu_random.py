@@ -134,3 +134,52 @@ def test_random_one_call_exact_topk(dev, oracle):
         assert buf[:nb].cpu().numpy().tobytes() == want.tobytes()
         assert gu.cpu().numpy().tobytes() == uu.tobytes()
     assert 1 in routes
+
+
+def test_random_write_step_across_the_selection_paths(dev, oracle):
+    """cx_ip_write_step on vector lengths on both sides of every limit between the selection paths (two
+    launches / chained passes / one candidate pass / single pass over both vectors), strided sample or
+    whole vector, three element types, inputs of several kinds, two residual-carrying steps each:
+    threshold, message and residual are the checker's."""
+    from comprex_amd.device import message_capacity
+    rng = np.random.default_rng(99)
+    np2t = {np.float32: torch.float32, np.float64: torch.float64, np.int32: torch.int32}
+    sizes = [1, 63, 4097, 40_960, 40_961, 100_000, 262_144, 262_145, 1 << 20, (1 << 22) + 1, (5 << 20) - 1, 5 << 20,
+             (1 << 23) + 1, (20 << 20) - 4, (20 << 20) + 4]
+    routes = set()
+    for case, n in enumerate(sizes + sizes):
+        dtype = [np.float32, np.float64, np.int32][case % 3]
+        if dtype == np.float64 and n > 12_000_000:
+            dtype = np.float32
+        topk = np.float32(rng.choice([0.0005, 0.01, 0.04, 0.1, 0.3]))
+        ds = 1000 if case % 4 == 3 else 1 << 30  # strided sample now and then, else the whole vector
+        kind = int(rng.integers(0, 4))
+        scale = 1000 if dtype == np.int32 else 1
+
+        def grad():
+            if kind == 0:
+                v = rng.standard_normal(n)
+            elif kind == 1:  # stretches of different scale
+                v = rng.standard_normal(n) * np.repeat(10.0 ** rng.uniform(-4, 0, n // 4096 + 1), 4096)[:n]
+            elif kind == 2:  # ties
+                v = np.round(rng.standard_normal(n) * 3)
+            else:            # mostly zeros
+                v = rng.standard_normal(n) * (rng.random(n) < 0.05)
+            return (v * scale).astype(dtype)
+
+        say("random write_step", case, dtype.__name__, n, float(topk), ds, kind)
+        r_h = np.zeros(n, dtype)
+        r = torch.zeros(n, dtype=np2t[dtype], device="cuda")
+        buf = torch.zeros(message_capacity(n, np2t[dtype]), dtype=torch.uint8, device="cuda")
+        thr_out = torch.zeros(1, dtype=np2t[dtype], device="cuda")
+        for _ in range(2):
+            g_h = grad()
+            g = torch.from_numpy(g_h).cuda()
+            nb = dev.write_step(buf, g, r, topk, ds, 10.0, d_thr=thr_out)
+            want_thr = oracle.topk_prepare_with(r_h, g_h, topk, ds, 10.0)
+            want = oracle.ip_compress(g_h, r_h, dtype(want_thr))
+            assert thr_out.cpu().numpy()[0] == dtype(want_thr), (case, n)
+            assert nb == want.size and buf[:nb].cpu().numpy().tobytes() == want.tobytes(), (case, n)
+            assert r.cpu().numpy().tobytes() == r_h.tobytes(), (case, n)
+        routes.add(dev.get_option("fused_topk_taken"))
+    assert 1 in routes or 2 in routes  # the single pass was among them
