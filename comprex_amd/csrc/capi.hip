@@ -603,13 +603,31 @@ int cx_ip_reduce(cx_handle h, cx_dtype dt, void* out, int out_n, const void* con
             return fail(CX_ERR_INVALID, "message %d must be a 4-byte aligned device pointer", r);
     if ((mode & CX_REDUCE_ANY_ORDER) && n_msgs > 0) {
         int sorted = 1;
-        CX_DISPATCH_RC(dt, messages_sorted<T>(h, msgs, n_msgs, &sorted));
+        long long pairs = 0;
+        CX_DISPATCH_RC(dt, messages_sorted<T>(h, msgs, n_msgs, &sorted, &pairs));
         if (!sorted) {
             // the reference's loop, message after message, pair after pair (src/compressor.hxx:640-658)
             if (!accumulate) CX_DISPATCH_RC(dt, launch_zero<T>(h, static_cast<T*>(out), out_n));
             for (int r = 0; r < n_msgs; ++r)
                 CX_DISPATCH_RC(dt, launch_sequential<T>(h, static_cast<T*>(out), out_n, msgs[r], 1));
             return CX_OK;
+        }
+        // Adding sparse messages into a long vector: one scatter per message touches the pairs' elements
+        // only, a pass over the vector reads and writes all of it.  Measured, fp32, 1 %-dense messages added
+        // into 64 Mi elements, 1 / 2 / 4 / 8 messages: 20.5 / 40.9 / 84.0 / 200 us as scatters against 83 /
+        // 88 / 93 / 94 us as one pass; into 16 Mi elements 4.7 / 10.2 / 23.2 / 45.6 against 24.0 / 25.6 /
+        // 28.4 / 33.6 us; into 1 Mi elements 4.5 / 7.0 / 12.5 / 23.1 against 7.0 / 7.1 / 8.1 / 10.3 us.  The
+        // model below (4.5 us a launch, 0.03 us per thousand pairs; 7 us + the vector's bytes twice at
+        // 6.5 TB/s) follows those figures; the pair count is known here because the order check read it.
+        if (accumulate && (mode & ~CX_REDUCE_ANY_ORDER) == 0 && h->reduce_variant == 0) {
+            const double elem_bytes = dt == CX_F64 ? 8.0 : 4.0;
+            const double scatter_us = 4.5 * n_msgs + 0.03e-3 * (double)pairs;
+            const double pass_us = 7.0 + 2.0 * elem_bytes * (double)out_n / 6.5e6;
+            if (scatter_us < pass_us) {
+                for (int r = 0; r < n_msgs; ++r)
+                    CX_DISPATCH_RC(dt, launch_add<T>(h, static_cast<T*>(out), out_n, msgs[r], 0));
+                return CX_OK;
+            }
         }
     }
     mode &= ~CX_REDUCE_ANY_ORDER;

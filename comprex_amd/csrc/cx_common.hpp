@@ -177,7 +177,8 @@ template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void*
 // the reference's loop, pair after pair: any index order, indices repeated anywhere (slow)
 template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, const void* msg, int add);
 // one pass over the messages' indices and one wait: *sorted = every message's indices ascend
-template <typename T> int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted);
+template <typename T>
+int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted, long long* total_pairs = nullptr);
 template <typename T>
 int launch_reduce(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int accumulate, int mode);
 int launch_copy_counted(cx_handle h, void* dst, const void* src, const int* d_bytes, long long capacity);

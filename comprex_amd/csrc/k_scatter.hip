@@ -130,10 +130,13 @@ __global__ __launch_bounds__(64) void sequential_kernel(T* out, int out_n,
 
 // *unsorted |= some message holds an index below its predecessor (or is made for a longer vector,
 // which the caller's path then reports).  grid.y = message.  The fast paths need ascending indices;
-// a caller that must take any order (the reference's loops do) asks first.
+// a caller that must take any order (the reference's loops do) asks first.  unsorted[1] += the
+// messages' pair counts (what the dispatch between a pass over the whole vector and one scatter per
+// message goes by).
 __global__ __launch_bounds__(kBlock) void order_check_kernel(MsgHeaders list, unsigned* __restrict__ unsorted, int pair_words) {
     const unsigned* msg = list.msg[blockIdx.y];
     const long long k = (long long)(int)msg[1];
+    if (blockIdx.x == 0 && threadIdx.x == 0 && k > 0) atomicAdd(unsorted + 1, (unsigned)k);
     const unsigned* pairs = msg + 2;
     const long long stride = (long long)gridDim.x * kBlock;
     bool bad = false;
@@ -1109,9 +1112,11 @@ template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, cons
 }
 
 // Are all the messages index-sorted?  One pass over their indices and one wait for the stream.
-template <typename T> int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted) {
+template <typename T>
+int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted, long long* total_pairs) {
     *sorted = 1;
-    unsigned* flag = reinterpret_cast<unsigned*>(h->d_status) + 16;  // a word of the status block
+    if (total_pairs) *total_pairs = 0;
+    unsigned* flag = reinterpret_cast<unsigned*>(h->d_status) + 16;  // two words of the status block: flag, pair count
     for (int first = 0; first < n_msgs; first += MsgHeaders::kMax) {
         MsgHeaders list;
         const int cnt = n_msgs - first < MsgHeaders::kMax ? n_msgs - first : MsgHeaders::kMax;
@@ -1121,12 +1126,11 @@ template <typename T> int messages_sorted(cx_handle h, const void* const* msgs, 
                            (int)Elem<T>::pair_words);
     }
     CX_HIP(hipGetLastError());
-    CX_HIP(hipMemcpyAsync(h->h_pinned + 13, flag, sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
+    CX_HIP(hipMemcpyAsync(h->h_pinned + 13, flag, 2 * sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
     CX_HIP(hipStreamSynchronize(h->stream));
-    if (h->h_pinned[13] != 0) {
-        *sorted = 0;
-        CX_HIP(hipMemsetAsync(flag, 0, sizeof(unsigned), h->stream));
-    }
+    if (h->h_pinned[13] != 0) *sorted = 0;
+    if (total_pairs) *total_pairs = (long long)(unsigned)h->h_pinned[14];
+    if (h->h_pinned[13] != 0 || h->h_pinned[14] != 0) CX_HIP(hipMemsetAsync(flag, 0, 2 * sizeof(unsigned), h->stream));
     return CX_OK;
 }
 
@@ -1202,7 +1206,7 @@ template int reserve_reduce<int>(cx_handle, int);
     template int launch_threshold_apply<T>(cx_handle, T*, T*, const T*, int, const T*, const T*); \
     template int launch_add<T>(cx_handle, T*, int, const void*, int);                             \
     template int launch_sequential<T>(cx_handle, T*, int, const void*, int);                      \
-    template int messages_sorted<T>(cx_handle, const void* const*, int, int*);                    \
+    template int messages_sorted<T>(cx_handle, const void* const*, int, int*, long long*);                    \
     template int launch_decompress<T>(cx_handle, T*, int, const void*);                           \
     template int launch_reduce<T>(cx_handle, T*, int, const void* const*, int, int, int);
 CX_INSTANTIATE(float)

@@ -768,6 +768,26 @@ def test_tiled_reduce_reports_unsorted_message(dev):
     assert e.value.code == _lib.CX_ERR_INDEX
 
 
+def test_any_order_accumulate_takes_scatters_or_one_pass_by_pair_count(dev, oracle):
+    """Adding index-sorted messages with CX_REDUCE_ANY_ORDER: the order check also reads the pair
+    counts, and few sparse messages are applied as one scatter each (only their elements are touched)
+    instead of one pass over the whole vector.  Both choices give the checker's sums, additions in
+    message order (half of each message's indices are shared with the others)."""
+    from comprex_amd import workloads as W
+    n = 6_000_000
+    for k, count in ((n // 2000, 3), (n // 20, 3), (n // 2000, 12)):
+        say("any-order accumulate", n, k, count)
+        msgs_h = W.c5_messages(seed=7 + k, n=n, ranks=count, k=k, shared=k // 2)
+        base = np.random.default_rng(k).standard_normal(n).astype(np.float32)
+        want = base.copy()
+        for m in msgs_h:
+            oracle.ip_add(m, want)
+        out = _gpu(base)
+        dev.reduce(out, [_gpu(m) for m in msgs_h], accumulate=True, mode=0, any_order=True)
+        dev.synchronize()
+        assert out.cpu().numpy().tobytes() == want.tobytes()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_add_and_reduce_take_any_index_order_when_asked(dev, oracle, dtype):
     """The reference's add walks the pairs as stored (src/compressor.hxx:640-658): any index order, an
