@@ -581,16 +581,14 @@ int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void*
 int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int check) {
     if (!h) return fail(CX_ERR_INVALID, "null handle");
     if (!msg || !aligned4(msg)) return fail(CX_ERR_INVALID, "message must be a 4-byte aligned device pointer");
+    // any index order: decided on the device, nothing waits (a message made for a longer vector is
+    // refused by the kernels themselves and reported with the status, like every other device-side error)
+    if (check == CX_ADD_ANY_ORDER) CX_DISPATCH(dt, launch_add_any_order<T>(h, static_cast<T*>(out), out_n, msg));
     if (check) {
         CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
         CX_HIP(hipStreamSynchronize(h->stream));
         if (h->h_pinned[8] > out_n)
             return fail(CX_ERR_MSG_TOO_LARGE, "Decompression vector size is bigger than output buffer!");
-    }
-    if (check == CX_ADD_ANY_ORDER) {
-        int sorted = 1;
-        CX_DISPATCH_RC(dt, messages_sorted<T>(h, &msg, 1, &sorted));
-        if (!sorted) CX_DISPATCH(dt, launch_sequential<T>(h, static_cast<T*>(out), out_n, msg, 1));
     }
     CX_DISPATCH(dt, launch_add<T>(h, static_cast<T*>(out), out_n, msg, 0));
 }

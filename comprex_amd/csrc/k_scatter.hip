@@ -41,8 +41,10 @@ __device__ __forceinline__ void atomic_accumulate(int* p, int v) { atomicAdd(p, 
 // OP 0: out[idx] = val (last pair of a run wins)   OP 1: out[idx] += val in order   OP 2: atomic +=
 template <typename T, int OP>
 __global__ __launch_bounds__(kBlock) void scatter_kernel(T* __restrict__ out, int out_n,
-                                                         const unsigned* __restrict__ msg, DeviceStatus* status) {
+                                                         const unsigned* __restrict__ msg, DeviceStatus* status,
+                                                         const unsigned* __restrict__ skip_if = nullptr) {
     constexpr int PW = Elem<T>::pair_words;
+    if (skip_if && *skip_if != 0u) return;  // the message is not index-sorted: the pair-after-pair kernel takes it
     const int n_msg = (int)msg[0];
     const long long k = (long long)(int)msg[1];
     if (n_msg > out_n) {
@@ -90,8 +92,20 @@ struct MsgHeaders {
 // Slow (tens of ns per pair): the fallback for messages the sorted paths refuse.
 template <typename T, int OP>
 __global__ __launch_bounds__(64) void sequential_kernel(T* out, int out_n,
-                                                       const unsigned* __restrict__ msg, DeviceStatus* status) {
+                                                       const unsigned* __restrict__ msg, DeviceStatus* status,
+                                                       unsigned* run_if = nullptr) {
     constexpr int PW = Elem<T>::pair_words;
+    if (run_if) {
+        // launched behind the order check and the sorted-path kernel: runs only when the check found the
+        // message unsorted (the sorted-path kernel then did nothing), and leaves the check's words clean
+        const unsigned unsorted = run_if[0];
+        __builtin_amdgcn_s_waitcnt(0);
+        if (threadIdx.x == 0) {
+            run_if[0] = 0u;
+            run_if[1] = 0u;
+        }
+        if (unsorted == 0u) return;
+    }
     const int n_msg = (int)msg[0];
     const long long k = (long long)(int)msg[1];
     if (n_msg > out_n) {
@@ -1111,6 +1125,24 @@ template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, cons
     return CX_OK;
 }
 
+// add_strategy for a message in ANY index order without the host in between: the order check, the
+// fast kernel (which does nothing when the check found disorder) and the pair-after-pair kernel (which
+// does nothing otherwise) are enqueued one behind the other.
+template <typename T> int launch_add_any_order(cx_handle h, T* out, int out_n, const void* msg) {
+    if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "add: bad arguments");
+    if (out_n == 0) return check_headers(h, &msg, 1);
+    unsigned* flag = reinterpret_cast<unsigned*>(h->d_status) + 16;
+    const unsigned* words = static_cast<const unsigned*>(msg);
+    MsgHeaders list;
+    for (int r = 0; r < MsgHeaders::kMax; ++r) list.msg[r] = r == 0 ? words : nullptr;
+    hipLaunchKernelGGL(order_check_kernel, dim3(256, 1), dim3(kBlock), 0, h->stream, list, flag, (int)Elem<T>::pair_words);
+    hipLaunchKernelGGL((scatter_kernel<T, 1>), dim3(grid_for(out_n, 1)), dim3(kBlock), 0, h->stream, out, out_n, words,
+                       h->d_status, flag);
+    hipLaunchKernelGGL((sequential_kernel<T, 1>), dim3(1), dim3(64), 0, h->stream, out, out_n, words, h->d_status, flag);
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
 // Are all the messages index-sorted?  One pass over their indices and one wait for the stream.
 template <typename T>
 int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted, long long* total_pairs) {
@@ -1206,7 +1238,8 @@ template int reserve_reduce<int>(cx_handle, int);
     template int launch_threshold_apply<T>(cx_handle, T*, T*, const T*, int, const T*, const T*); \
     template int launch_add<T>(cx_handle, T*, int, const void*, int);                             \
     template int launch_sequential<T>(cx_handle, T*, int, const void*, int);                      \
-    template int messages_sorted<T>(cx_handle, const void* const*, int, int*, long long*);                    \
+    template int messages_sorted<T>(cx_handle, const void* const*, int, int*, long long*);     \
+    template int launch_add_any_order<T>(cx_handle, T*, int, const void*);                    \
     template int launch_decompress<T>(cx_handle, T*, int, const void*);                           \
     template int launch_reduce<T>(cx_handle, T*, int, const void* const*, int, int, int);
 CX_INSTANTIATE(float)

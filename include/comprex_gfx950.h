@@ -251,13 +251,15 @@ int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void*
 
 /* CompressorIndexPairs<T>::add_strategy (src/compressor.hxx:640-658): out[index] += value
  * in message order.  A message whose n exceeds out_n changes nothing and records
- * CX_ERR_MSG_TOO_LARGE.  `check` != 0 reads the header first and returns that error
+ * CX_ERR_MSG_TOO_LARGE.  `check` == 1 reads the header first and returns that error
  * synchronously, as the reference throws before touching `out`.
  * Index order: the kernel applies a run of equal NEIGHBOURING indices in message order, which is
  * all an index-sorted message (what the compressors emit) needs; an index below its predecessor
  * records CX_ERR_INDEX, because equal indices may then lie apart and `out` is no longer what the
- * reference's loop gives.  check == CX_ADD_ANY_ORDER looks at the indices first (one pass, one more
- * wait) and applies a message that is not sorted pair after pair, exactly as the reference does. */
+ * reference's loop gives.  check == CX_ADD_ANY_ORDER takes any order, exactly as the reference does,
+ * and waits for nothing: a pass over the indices, the fast kernel and the pair-after-pair kernel are
+ * enqueued one behind the other and the device decides which of the two does the work; errors
+ * (the oversize message included) come with the status, as from any asynchronous call. */
 enum { CX_ADD_ANY_ORDER = 2 };
 int cx_ip_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int check);
 
