@@ -181,6 +181,16 @@ int rle_compress_impl(cx_handle h, void* out_msg, long long out_capacity, const 
 
 template <typename T>
 int decompress_impl(cx_handle h, void* out, int out_n, const void* msg, int* h_bytes) {
+    if (h_bytes && (h->reduce_variant == 0 || h->reduce_variant == 2)) {
+        // the reporting form takes any index order, as the reference does (src/compressor.hxx:613-633):
+        // decided on the device, one wait at the end
+        int rc_any = launch_decompress_any_order<T>(h, static_cast<T*>(out), out_n, msg);
+        if (rc_any != CX_OK) return rc_any;
+        CX_HIP(hipMemcpyAsync(h->h_pinned + 8, msg, 8, hipMemcpyDeviceToHost, h->stream));
+        rc_any = collect_status(h);
+        *h_bytes = 8 + h->h_pinned[9] * 4 * Elem<T>::pair_words;
+        return rc_any;
+    }
     if (h_bytes) {
         // what earlier calls left behind is reported now, so that the status read below belongs to
         // this message alone (a message cut short by an earlier compress is not this call's business)

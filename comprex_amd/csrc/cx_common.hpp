@@ -175,6 +175,7 @@ template <typename T> int launch_rle_decode(cx_handle h, T* out, int out_n, cons
 template <typename T> int launch_decompress(cx_handle h, T* out, int out_n, const void* msg);
 template <typename T> int launch_add(cx_handle h, T* out, int out_n, const void* msg, int atomic);
 template <typename T> int launch_add_any_order(cx_handle h, T* out, int out_n, const void* msg);
+template <typename T> int launch_decompress_any_order(cx_handle h, T* out, int out_n, const void* msg);
 // the reference's loop, pair after pair: any index order, indices repeated anywhere (slow)
 template <typename T> int launch_sequential(cx_handle h, T* out, int out_n, const void* msg, int add);
 // one pass over the messages' indices and one wait: *sorted = every message's indices ascend

@@ -182,9 +182,11 @@ struct MsgList {
 // t in [0, ntiles]; blockIdx.y selects the message.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void bounds_kernel(MsgList list, int out_n, unsigned ntiles,
-                                                        unsigned* __restrict__ bounds, DeviceStatus* status) {
+                                                        unsigned* __restrict__ bounds, DeviceStatus* status,
+                                                        const unsigned* __restrict__ skip_if) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kReduceTile = ReduceTile<T>::value;
+    if (skip_if && *skip_if != 0u) return;  // an order check in front found disorder: the pair-after-pair kernels take over
     const int r = blockIdx.y;
     const unsigned* msg = list.msg[r];
     const int n_msg = (int)msg[0];
@@ -220,11 +222,12 @@ __global__ __launch_bounds__(kBlock) void bounds_kernel(MsgList list, int out_n,
 template <typename T, int OP, bool ACCUM, int RMAX>
 __global__ __launch_bounds__(kBlock) void tiled_kernel(T* __restrict__ out, int out_n, MsgList list, int n_msgs,
                                                        unsigned ntiles, const unsigned* __restrict__ bounds,
-                                                       DeviceStatus* status) {
+                                                       DeviceStatus* status, const unsigned* __restrict__ skip_if) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int VEC = 16 / (int)sizeof(T);
     constexpr int kReduceTile = ReduceTile<T>::value;
     __shared__ T tile[kReduceTile];
+    if (skip_if && *skip_if != 0u) return;
     const int tid = threadIdx.x, lane = tid & 63;
     const unsigned t = blockIdx.x;
     const long long base = (long long)t * kReduceTile;
@@ -882,7 +885,8 @@ int check_headers(cx_handle h, const void* const* msgs, int n_msgs) {
 }
 
 template <typename T>
-int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate);
+int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate,
+                 const unsigned* skip_if = nullptr);
 
 template <typename T>
 int launch_merged(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
@@ -934,7 +938,8 @@ int ensure_bounds(cx_handle h, size_t need) {
 }
 
 template <typename T>
-int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate) {
+int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_msgs, int op, int accumulate,
+                 const unsigned* skip_if) {
     if (out_n == 0) return check_headers(h, msgs, n_msgs);
     constexpr int kReduceTile = ReduceTile<T>::value;
     const unsigned ntiles = (unsigned)(((long long)out_n + kReduceTile - 1) / kReduceTile);
@@ -949,12 +954,12 @@ int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_
             if (grid < 1) grid = 1;
             if (grid > 1024) grid = 1024;
             hipLaunchKernelGGL(bounds_kernel<T>, dim3(grid, cnt), dim3(kBlock), 0, h->stream, list, out_n, ntiles,
-                               h->reduce_bounds, h->d_status);
+                               h->reduce_bounds, h->d_status, skip_if);
         }
         const bool acc = accumulate || first > 0;
 #define CX_TILED(OP, ACC, RMAX)                                                                                     \
     hipLaunchKernelGGL((tiled_kernel<T, OP, ACC, RMAX>), dim3(ntiles), dim3(kBlock), 0, h->stream, out, out_n, list, \
-                       cnt, ntiles, h->reduce_bounds, h->d_status)
+                       cnt, ntiles, h->reduce_bounds, h->d_status, skip_if)
         if (op == 0) CX_TILED(0, false, 1);
         else if (cnt <= 8) { if (acc) CX_TILED(1, true, 8); else CX_TILED(1, false, 8); }
         else { if (acc) CX_TILED(1, true, kMaxMsgs); else CX_TILED(1, false, kMaxMsgs); }
@@ -966,7 +971,9 @@ int launch_tiled(cx_handle h, T* out, int out_n, const void* const* msgs, int n_
 }
 
 template <typename T, int VEC>
-__global__ __launch_bounds__(kBlock) void zero_kernel(T* __restrict__ v, long long n) {
+__global__ __launch_bounds__(kBlock) void zero_kernel(T* __restrict__ v, long long n,
+                                                      const unsigned* __restrict__ run_if = nullptr) {
+    if (run_if && *run_if == 0u) return;
     const long long stride = (long long)gridDim.x * kBlock;
     const long long nvec = n / VEC;
     Pack<T, VEC> z;
@@ -1143,6 +1150,30 @@ template <typename T> int launch_add_any_order(cx_handle h, T* out, int out_n, c
     return CX_OK;
 }
 
+// decompression_strategy for a message in ANY index order without the host in between: order check, the
+// tiled kernels (which do nothing when the check found disorder), then zero fill and the pair-after-pair
+// kernel (which do nothing otherwise).
+template <typename T> int launch_decompress_any_order(cx_handle h, T* out, int out_n, const void* msg) {
+    if ((!out && out_n > 0) || !msg || out_n < 0) return fail(CX_ERR_INVALID, "decompress: bad arguments");
+    if (out_n == 0) return check_headers(h, &msg, 1);
+    unsigned* flag = reinterpret_cast<unsigned*>(h->d_status) + 16;
+    const unsigned* words = static_cast<const unsigned*>(msg);
+    MsgHeaders list;
+    for (int r = 0; r < MsgHeaders::kMax; ++r) list.msg[r] = r == 0 ? words : nullptr;
+    hipLaunchKernelGGL(order_check_kernel, dim3(256, 1), dim3(kBlock), 0, h->stream, list, flag, (int)Elem<T>::pair_words);
+    int rc = launch_tiled<T>(h, out, out_n, &msg, 1, 0, 0, flag);
+    if (rc != CX_OK) return rc;
+    constexpr int kVec = 16 / (int)sizeof(T);
+    if ((reinterpret_cast<uintptr_t>(out) & 15u) == 0)
+        hipLaunchKernelGGL((zero_kernel<T, kVec>), dim3(grid_for(out_n, 4 * kVec)), dim3(kBlock), 0, h->stream, out,
+                           (long long)out_n, flag);
+    else
+        hipLaunchKernelGGL((zero_kernel<T, 1>), dim3(grid_for(out_n, 4)), dim3(kBlock), 0, h->stream, out, (long long)out_n, flag);
+    hipLaunchKernelGGL((sequential_kernel<T, 0>), dim3(1), dim3(64), 0, h->stream, out, out_n, words, h->d_status, flag);
+    CX_HIP(hipGetLastError());
+    return CX_OK;
+}
+
 // Are all the messages index-sorted?  One pass over their indices and one wait for the stream.
 template <typename T>
 int messages_sorted(cx_handle h, const void* const* msgs, int n_msgs, int* sorted, long long* total_pairs) {
@@ -1239,7 +1270,8 @@ template int reserve_reduce<int>(cx_handle, int);
     template int launch_add<T>(cx_handle, T*, int, const void*, int);                             \
     template int launch_sequential<T>(cx_handle, T*, int, const void*, int);                      \
     template int messages_sorted<T>(cx_handle, const void* const*, int, int*, long long*);     \
-    template int launch_add_any_order<T>(cx_handle, T*, int, const void*);                    \
+    template int launch_add_any_order<T>(cx_handle, T*, int, const void*);                        \
+    template int launch_decompress_any_order<T>(cx_handle, T*, int, const void*);                    \
     template int launch_decompress<T>(cx_handle, T*, int, const void*);                           \
     template int launch_reduce<T>(cx_handle, T*, int, const void* const*, int, int, int);
 CX_INSTANTIATE(float)
