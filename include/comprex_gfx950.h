@@ -244,9 +244,10 @@ int cx_rle_add(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg);
  * Index order: the compressors of this library and of the reference emit ascending indices, and
  * the fast path requires them (an index below its predecessor records CX_ERR_INDEX).  The
  * reference's decoder takes any order, repeats anywhere, last value wins: with h_bytes != NULL
- * (the call waits anyway) such a message is decoded once more, pair after pair, with exactly that
- * result; with h_bytes == NULL the error stands.  Indices outside [0, out_n) are CX_ERR_INDEX
- * either way (the reference writes out of bounds). */
+ * a pass over the indices runs first and the device decides between the fast kernels and the
+ * pair-after-pair kernel, with exactly that result (one wait, at the end, for the byte count and
+ * the status); with h_bytes == NULL the fast path runs alone and the error stands.  Indices outside
+ * [0, out_n) are CX_ERR_INDEX either way (the reference writes out of bounds). */
 int cx_ip_decompress(cx_handle h, cx_dtype dt, void* out, int out_n, const void* msg, int* h_bytes);
 
 /* CompressorIndexPairs<T>::add_strategy (src/compressor.hxx:640-658): out[index] += value
