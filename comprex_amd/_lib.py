@@ -53,6 +53,7 @@ def lib():
         "cx_synchronize": (i, [vp]),
         "cx_get_stream": (vp, [vp]),
         "cx_stream_create": (i, [C.POINTER(vp)]),
+        "cx_stream_create_blocking": (i, [C.POINTER(vp)]),
         "cx_stream_destroy": (i, [vp]),
         "cx_stream_synchronize": (i, [vp]),
         "cx_event_create": (i, [C.POINTER(vp)]),

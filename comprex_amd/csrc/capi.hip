@@ -362,6 +362,16 @@ int cx_stream_create(void** out_stream) {
     return CX_OK;
 }
 
+int cx_stream_create_blocking(void** out_stream) {
+    if (!out_stream) return fail(CX_ERR_INVALID, "cx_stream_create_blocking: null output");
+    *out_stream = nullptr;
+    if (cx_device_count() < 1) return fail(CX_ERR_HIP, "cx_stream_create_blocking: no HIP device available");
+    hipStream_t s = nullptr;
+    CX_HIP(hipStreamCreateWithFlags(&s, hipStreamDefault));  // default priority
+    *out_stream = static_cast<void*>(s);
+    return CX_OK;
+}
+
 int cx_stream_destroy(void* hip_stream) {
     if (hip_stream) CX_HIP(hipStreamDestroy(static_cast<hipStream_t>(hip_stream)));
     return CX_OK;

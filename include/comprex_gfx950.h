@@ -102,9 +102,13 @@ void* cx_get_stream(cx_handle h);
  * plain host code).  The reference's RDMA put is asynchronous and its receiver waits for a
  * notification (src/comprEx.tpp:190,231,243): here every ComprEx object works on a stream of its
  * own and a message's hand-over is an event the sender records and the receiver's stream waits
- * for.  Streams are created non-blocking (no implicit ordering with the null stream) and at the
- * default priority; events carry no timing.  A NULL stream argument names the null stream. */
+ * for.  cx_stream_create makes a non-blocking stream (no implicit ordering with the null stream),
+ * cx_stream_create_blocking one the runtime orders with the null stream (what the objects use);
+ * both at the default priority; events carry no timing.  A NULL stream argument names the null stream. */
 int cx_stream_create(void** out_stream);
+/* A stream that IS ordered with the null stream, both ways, by the runtime (a "blocking" stream): what an
+ * object whose caller works on the null stream needs, without an event join around every call. */
+int cx_stream_create_blocking(void** out_stream);
 int cx_stream_destroy(void* hip_stream);
 int cx_stream_synchronize(void* hip_stream);
 int cx_event_create(void** out_event);
