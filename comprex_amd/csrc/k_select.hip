@@ -602,6 +602,119 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
     }
 }
 
+// ---- up to one block's worth of keys: ONE launch -------------------------------------------
+// ThresholdTopK's default is 1000 strided samples (src/threshold.hxx:130,182-186), so this is what an
+// ordinary writeRemote runs: the block gathers its keys straight into LDS and finishes there (digits
+// from the first bit in which the keys differ, then direct ranking of the last few), instead of one
+// launch that stores the keys and a second that reads them back.
+template <typename T, int SMODE, bool HAS_ADD>
+__global__ __launch_bounds__(kFinishBlock) void select_one_block_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                                        const int* __restrict__ idx, int m, int n,
+                                                                        float stepsize, unsigned long long rank,
+                                                                        int plus_one, T* __restrict__ thr_out,
+                                                                        unsigned* __restrict__ zero_word) {
+    using key_t = typename Elem<T>::key_t;
+    constexpr int kKeyBits = Elem<T>::key_bits;
+    constexpr key_t kAllBits = (key_t)(~(key_t)0) >> (8 * (int)sizeof(key_t) - kKeyBits);
+    __shared__ __align__(8) unsigned lds_hist[kRadixBins];
+    __shared__ key_t s_list[kFinishBlock];
+    __shared__ key_t s_and, s_or, s_answer;
+    __shared__ unsigned s_digit, s_fill;
+    __shared__ unsigned long long s_above, s_sum[kFinishBlock / 64];
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    if (t == 0) {
+        s_and = kAllBits;
+        s_or = (key_t)0;
+    }
+    if (zero_word && t == 0) *zero_word = 0u;
+    __syncthreads();
+    const bool have = t < m;
+    key_t mine = 0;
+    if (have) {
+        long long p;
+        bool ok = true;
+        if (SMODE == 0) {
+            p = t;
+        } else if (SMODE == 1) {
+            p = (long long)(int)__fmul_rn((float)t, stepsize);  // (int)(i * stepsize), product in fp32
+            if (p > (long long)n - 1) p = (long long)n - 1;     // the reference would read out of bounds
+            if (p < 0) p = 0;
+        } else {
+            p = idx[t];
+            ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
+            if (!ok) p = 0;
+        }
+        T v = vec[p];
+        if (HAS_ADD) v = (T)(v + add[p]);
+        mine = ok ? key_of(v) : (key_t)0;
+        s_list[t] = mine;
+    }
+    key_t all_and = have ? mine : kAllBits, all_or = have ? mine : (key_t)0;
+    wave_and_or<key_t>(all_and, all_or);
+    if (lane == 0) {
+        atomicAnd(&s_and, all_and);
+        atomicOr(&s_or, all_or);
+    }
+    __syncthreads();
+    const unsigned list_n = (unsigned)m;
+    const key_t differ = s_and ^ s_or;
+    int lo = differ ? 64 - __clzll((unsigned long long)differ) : 0;  // the bits below this one are still open
+    const key_t open_bits = lo >= 8 * (int)sizeof(key_t) ? (key_t)~(key_t)0 : (key_t)(((key_t)1 << lo) - 1);
+    key_t mask = kAllBits & ~open_bits;
+    key_t prefix = s_and & mask;
+    while (lo > 0) {
+        const int bits = lo < kRadixBits ? lo : kRadixBits;
+        const int shift = lo - bits;
+        const unsigned digit_mask = (1u << bits) - 1u;
+        for (int b = t; b < kRadixBins; b += kFinishBlock) lds_hist[b] = 0u;
+        __syncthreads();
+        if (have && (mine & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(mine >> shift) & digit_mask], 1u);
+        __syncthreads();
+        unsigned digit;
+        unsigned long long above;
+        block_pick<kFinishBlock>(lds_hist, rank, s_sum, &s_digit, &s_above, digit, above);
+        const unsigned in_digit = lds_hist[digit];
+        prefix |= (key_t)digit << shift;
+        mask |= (key_t)((1ull << bits) - 1ull) << shift;
+        rank -= above;
+        lo = shift;
+        if (lo == 0) break;
+        __syncthreads();
+        if (in_digit <= (unsigned)kDirect && in_digit > 0u) {
+            // few keys left: the wanted one has at most `rank` keys above it and more than `rank` at or above it
+            key_t* cand = reinterpret_cast<key_t*>(lds_hist);
+            if (t == 0) {
+                s_fill = 0u;
+                s_answer = prefix;
+            }
+            __syncthreads();
+            if (have && (mine & mask) == prefix) cand[atomicAdd(&s_fill, 1u)] = mine;
+            __syncthreads();
+            const unsigned c = s_fill;  // == in_digit
+            if ((unsigned)t < c) {
+                const key_t me = cand[t];
+                unsigned gt = 0, ge = 0;
+                for (unsigned j = 0; j < c; ++j) {
+                    const key_t x = cand[j];
+                    gt += x > me ? 1u : 0u;
+                    ge += x >= me ? 1u : 0u;
+                }
+                if ((unsigned long long)gt <= rank && rank < (unsigned long long)ge) s_answer = me;
+            }
+            __syncthreads();
+            prefix = s_answer;
+            lo = 0;
+        }
+    }
+    (void)list_n;
+    if (t == 0) {
+        T v = value_of(prefix, T());
+        if (plus_one) v = (T)(v + 1);
+        *thr_out = v;
+    }
+}
+
 // ---- whole-vector selection with a sampled lower bound ---------------------------------
 // Copies every key >= the key of *d_bound into `cand` (order irrelevant).  Each wavefront
 // gathers its matches in an LDS segment and appends the segment with ONE global atomic when it
@@ -846,6 +959,23 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
     // keys (two dependent gathers per key and pass) and 8-byte keys (six passes) stay with the two launches.
     const bool two_launches = m <= kSmallSelect && (sample_mode != kSampleFull || kPasses > 3 || zero_word ||
                                                      m <= 40960 || (short_k > 0 && rank <= 1500ull));
+    if (two_launches && m <= kFinishBlock) {
+#define CX_ONE(SM, HA)                                                                                              \
+    hipLaunchKernelGGL((select_one_block_kernel<T, SM, HA>), dim3(1), dim3(kFinishBlock), 0, h->stream, vec, add_vec, \
+                       d_idx, m, n, stepsize, rank, plus_one, d_thr_out, zero_word)
+#define CX_ONE_MODE(HA)                                      \
+    do {                                                     \
+        if (sample_mode == kSampleFull) CX_ONE(0, HA);       \
+        else if (sample_mode == kSampleStrided) CX_ONE(1, HA); \
+        else CX_ONE(2, HA);                                  \
+    } while (0)
+        if (add_vec) CX_ONE_MODE(true);
+        else CX_ONE_MODE(false);
+#undef CX_ONE_MODE
+#undef CX_ONE
+        CX_HIP(hipGetLastError());
+        return CX_OK;
+    }
     if (two_launches) {
         int rc_keys = ensure_select_keys(h);
         if (rc_keys != CX_OK) return rc_keys;

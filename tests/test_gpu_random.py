@@ -94,6 +94,41 @@ def test_random_thresholds_every_sampling_rule(dev, oracle):
         assert dev.topk_threshold(gv, None, topk, ds, 10.0) == oracle.topk_prepare(v, topk, ds, 10.0)
 
 
+def test_random_thresholds_from_at_most_one_block_of_keys(dev, oracle):
+    """Up to 1024 keys (ThresholdTopK's default is 1000 strided samples, src/threshold.hxx:130) are
+    selected by one launch of one block: every sampling rule, lengths from 1 on, ties, all-zero and
+    constant-magnitude vectors, top-k fractions from one key to all of them."""
+    rng = np.random.default_rng(5)
+    for case in range(240):
+        dtype = DTYPES[case % 3]
+        n = int(rng.choice([1, 2, 5, 63, 64, 65, 255, 256, 257, 1000, 1023, 1024, 1025, 5000, 61706, 1_000_003]))
+        kind = int(rng.integers(0, 5))
+        if kind == 0:
+            v = rng.standard_normal(n)
+        elif kind == 1:
+            v = np.round(rng.standard_normal(n) * 2)
+        elif kind == 2:
+            v = rng.standard_normal(n) * (rng.random(n) < 0.05)
+        elif kind == 3:
+            v = np.zeros(n)
+        else:
+            v = np.full(n, 3.0) * rng.choice([-1, 1], n)
+        if dtype == np.int32:
+            v = v * 1000
+        v = v.astype(dtype)
+        a = (rng.standard_normal(n) * (10 if dtype == np.int32 else 0.01)).astype(dtype)
+        topk = np.float32(rng.choice([0.0001, 0.001, 0.01, 0.1, 0.5, 0.999, 1.0]))
+        ds = int(rng.choice([1, 7, 100, 1000, 1024]))
+        m = int(rng.integers(1, 1025))
+        idx = rng.integers(0, n, m).astype(np.int32)
+        say("random one-block threshold", case, dtype.__name__, n, kind, float(topk), ds, m)
+        gv, ga = torch.from_numpy(v).cuda(), torch.from_numpy(a).cuda()
+        assert dev.topk_threshold(gv, ga, topk, ds, 10.0) == oracle.topk_prepare_with(v, a, topk, ds, 10.0)
+        assert dev.topk_threshold(gv, None, topk, ds, 10.0) == oracle.topk_prepare(v, topk, ds, 10.0)
+        assert dev.topk_threshold_indexed(gv, ga, torch.from_numpy(idx).cuda(), topk) == \
+            oracle.topk_prepare_indexed(v, a, idx, topk)
+
+
 def test_random_one_call_exact_topk(dev, oracle):
     from comprex_amd.device import message_capacity
     rng = np.random.default_rng(2024)
