@@ -488,7 +488,7 @@ def main():
                                       ("C3", W.C3, W.c3_gradient, 3)):
                 extra["configs"][key] = config_leg(torch, W, cfg, fn, min(args.cpu_seconds, 5.0), not args.no_cpu, cap)
             extra["configs"]["launches_per_step"] = {
-                "C1": 6, "C2": 6, "C3": 9,
+                "C1": 5, "C2": 5, "C3": 9,
                 "source": "rocprofv3 kernel trace of these legs, profiles/configs_C1_C2_C3_kernel_trace.txt, not this run"}
 
         # reduce: 8 simulated ranks' 1 %-dense messages into a 64 Mi dense vector (config C5)

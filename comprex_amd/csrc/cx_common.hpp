@@ -127,6 +127,16 @@ struct cx_handle_s {
     int select_short_list = 1;         // 1 = the two-launch select passes a short list of top keys to its second launch
     int fused_topk = 1;                // cx_ip_compress_topk's single-pass route: 0 never, 1 from 20 Mi elements, 2 from 2^23
     int fused_topk_taken = 0;          // how the last cx_ip_compress_topk ran: 0 two calls, 1 single pass, 2 single pass abandoned
+    // A chained whole-vector selection whose last pick is left to the compress pass that follows it
+    // (launch_compress_topk asks for this with defer_pick): that pass's blocks pick from the last
+    // histogram themselves, which spares the launch of a one-block kernel.
+    bool defer_pick = false;
+    struct {
+        bool active = false;
+        unsigned long long rank = 0;
+        int plus_one = 0;
+        void* thr_out = nullptr;
+    } pending_pick;
     int reduce_variant = 0;            // 0 = rank-ordered, kernel chosen by message count; 1 = per-message scatter;
                                        // 2 = always one block per tile behind a bounds pass; 3 = always the pipelined kernel
     int reduce_blocks_per_cu = 1;      // persistent blocks per compute unit of the merged reduce
@@ -147,6 +157,8 @@ int locate_static_scratch(unsigned** out);
 // Pre-size a module's scratch for vectors of up to n elements of T, so that later calls find it large enough.
 template <typename T> int reserve_compact(cx_handle h, int n);
 template <typename T> int reserve_select(cx_handle h, int n);
+// makes the pick a selection left pending (handle's pending_pick) with a launch of its own
+template <typename T> int launch_pending_pick(cx_handle h);
 template <typename T> int reserve_reduce(cx_handle h, int n);
 template <typename T> int reserve_rle(cx_handle h, int n);
 long long noalloc_max_elements();

@@ -252,26 +252,15 @@ __device__ __forceinline__ unsigned process_tile(const T* __restrict__ data, T* 
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
-__global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
-                                                       const T* __restrict__ thr_ptr, T thr_val,
-                                                       unsigned* __restrict__ staging, unsigned* __restrict__ counts,
-                                                       unsigned* __restrict__ block_sums,
-                                                       unsigned* __restrict__ redo_flag, unsigned epoch,
-                                                       unsigned ntiles, int reverse, unsigned cached_from,
-                                                       unsigned slot_pairs) {
-    // survivors of this block's tiles, summed in LDS; the wavefront that finishes last stores
-    // the sum, which spares the gather kernel a scan over every tile count
-    __shared__ unsigned s_sum, s_done;
-    if (threadIdx.x == 0) {
-        s_sum = 0u;
-        s_done = 0u;
-    }
-    __syncthreads();
+__device__ __forceinline__ void stage_block(const T* __restrict__ data, T* __restrict__ update, long long n, const T thr,
+                                            unsigned* __restrict__ staging, unsigned* __restrict__ counts,
+                                            unsigned* __restrict__ block_sums, unsigned* __restrict__ redo_flag,
+                                            unsigned epoch, unsigned ntiles, int reverse, unsigned cached_from,
+                                            unsigned slot_pairs, unsigned& s_sum, unsigned& s_done) {
     // reversed launches walk the blocks from the end: they start on what the previous pass left cached
     const unsigned block = reverse ? gridDim.x - 1u - blockIdx.x : blockIdx.x;
     const unsigned tile = block * kWavesPerBlock + (threadIdx.x >> 6);
     if (tile >= ntiles) return;
-    const T thr = thr_ptr ? *thr_ptr : thr_val;
     // Only the last part of the walk can still be in the memory-side cache when the next launch
     // starts there: that part of the residual is read cacheably, everything before it bypasses the
     // caches like the gradient (a read that allocates pushes out lines that then have to be written
@@ -292,6 +281,58 @@ __global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ dat
         if (atomicAdd(&s_done, 1u) == tiles_here - 1u)
             reinterpret_cast<unsigned short*>(block_sums)[block] = (unsigned short)atomicAdd(&s_sum, 0u);
     }
+}
+
+template <typename T, int MODE, int VEC, int ITEMS>
+__global__ __launch_bounds__(kBlock) void stage_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
+                                                       const T* __restrict__ thr_ptr, T thr_val,
+                                                       unsigned* __restrict__ staging, unsigned* __restrict__ counts,
+                                                       unsigned* __restrict__ block_sums,
+                                                       unsigned* __restrict__ redo_flag, unsigned epoch,
+                                                       unsigned ntiles, int reverse, unsigned cached_from,
+                                                       unsigned slot_pairs) {
+    // survivors of this block's tiles, summed in LDS; the wavefront that finishes last stores
+    // the sum, which spares the gather kernel a scan over every tile count
+    __shared__ unsigned s_sum, s_done;
+    if (threadIdx.x == 0) {
+        s_sum = 0u;
+        s_done = 0u;
+    }
+    __syncthreads();
+    const T thr = thr_ptr ? *thr_ptr : thr_val;
+    stage_block<T, MODE, VEC, ITEMS>(data, update, n, thr, staging, counts, block_sums, redo_flag, epoch, ntiles, reverse,
+                                     cached_from, slot_pairs, s_sum, s_done);
+}
+
+// The same pass behind a chained radix selection (k_select.hip) whose last pick has not been made: every
+// block makes it for itself from the last pass's complete histogram, as the blocks of a chained pass do,
+// so the one-block kernel that would only pick and store the threshold is not launched.  Block 0 stores
+// the threshold for the kernels that follow (gather_kernel reads it, and clears the histograms).
+template <typename T, int MODE, int VEC, int ITEMS>
+__global__ __launch_bounds__(kBlock) void stage_pick_kernel(const T* __restrict__ data, T* __restrict__ update, long long n,
+                                                            const SelectState* __restrict__ sel, unsigned long long rank0,
+                                                            int plus_one, T* __restrict__ thr_out,
+                                                            unsigned* __restrict__ staging, unsigned* __restrict__ counts,
+                                                            unsigned* __restrict__ block_sums,
+                                                            unsigned* __restrict__ redo_flag, unsigned epoch,
+                                                            unsigned ntiles, int reverse, unsigned cached_from,
+                                                            unsigned slot_pairs) {
+    constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
+    using key_t = typename Elem<T>::key_t;
+    __shared__ unsigned s_sum, s_done;
+    __shared__ unsigned lds_hist[kRadixBins];
+    __shared__ unsigned s_digit;
+    __shared__ unsigned long long s_above, s_part[kBlock / 64];
+    if (threadIdx.x == 0) {
+        s_sum = 0u;
+        s_done = 0u;
+    }
+    const PickState picked = state_entering_pass<T, kBlock>(sel, kPasses, rank0, lds_hist, s_part, &s_digit, &s_above);
+    T thr = value_of((key_t)picked.prefix, T());
+    if (plus_one) thr = (T)(thr + 1);
+    if (blockIdx.x == 0 && threadIdx.x == 0) *thr_out = thr;
+    stage_block<T, MODE, VEC, ITEMS>(data, update, n, thr, staging, counts, block_sums, redo_flag, epoch, ntiles, reverse,
+                                     cached_from, slot_pairs, s_sum, s_done);
 }
 
 template <typename T, int MODE, int VEC, int ITEMS>
@@ -324,7 +365,8 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     const T* __restrict__ data, T* __restrict__ update, long long n, const T* __restrict__ thr_ptr, T thr_val,
     const unsigned* __restrict__ counts, const unsigned* __restrict__ block_sums, unsigned* __restrict__ offsets,
     const unsigned* __restrict__ staging, unsigned ntiles, unsigned* __restrict__ msg_words, long long cap_pairs,
-    int* __restrict__ size_prefix, int inline_redo, DeviceStatus* status, unsigned slot_pairs) {
+    int* __restrict__ size_prefix, int inline_redo, DeviceStatus* status, unsigned slot_pairs,
+    unsigned* __restrict__ zero_words, unsigned zero_count) {
     constexpr int PW = Elem<T>::pair_words;
     constexpr int kWaves = kGatherBlock / 64;
     // pairs a lane moves per round: searches and loads of one round are independent
@@ -332,6 +374,12 @@ __global__ __launch_bounds__(kGatherBlock) void gather_kernel(
     __shared__ unsigned s_before[kWaves];
     __shared__ unsigned s_off[65];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // words a kernel before this one has finished with (a selection's histograms), cleared for their next
+    // use by one block more than the tiles need
+    if (zero_words && blockIdx.x * kGatherTiles >= ntiles) {
+        for (unsigned b = tid; b < zero_count; b += kGatherBlock) zero_words[b] = 0u;
+        return;
+    }
 
     // Order of the loads: the tiles' counts first, then (their scan known) the staged pairs of the first
     // round, and only then the sums of the streaming blocks before this block's tiles, which give the
@@ -575,15 +623,34 @@ int launch_all(cx_handle h, const T* data, T* update, int n, const T* thr_ptr, T
         h->profile_count += 1;
         CX_HIP(hipEventRecord(ev[0], h->stream));
     }
-    hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
-                       (long long)n, thr_ptr, thr_val, sc.staging, sc.counts, sc.block_sums, redo_flag, h->epoch, ntiles,
-                       reverse, cached_from, slot_pairs);
+    unsigned* zero_words = nullptr;
+    unsigned zero_count = 0u;
+    bool picked_here = false;
+    if constexpr (MODE == 0) {
+        if (h->pending_pick.active) {
+            // the selection before this call left its last pick to this pass (see stage_pick_kernel)
+            constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
+            h->pending_pick.active = false;
+            picked_here = true;
+            zero_words = &h->sel->pass_hist[0][0];
+            zero_count = (unsigned)((kPasses + 1) * kRadixBins);
+            hipLaunchKernelGGL((stage_pick_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data,
+                               update, (long long)n, h->sel, h->pending_pick.rank, h->pending_pick.plus_one,
+                               static_cast<T*>(h->pending_pick.thr_out), sc.staging, sc.counts, sc.block_sums, redo_flag,
+                               h->epoch, ntiles, reverse, cached_from, slot_pairs);
+        }
+    }
+    if (!picked_here)
+        hipLaunchKernelGGL((stage_kernel<T, MODE, VEC, ITEMS>), dim3(stage_blocks), dim3(kBlock), 0, h->stream, data, update,
+                           (long long)n, thr_ptr, thr_val, sc.staging, sc.counts, sc.block_sums, redo_flag, h->epoch, ntiles,
+                           reverse, cached_from, slot_pairs);
     if (ev) CX_HIP(hipEventRecord(ev[1], h->stream));
     const unsigned gather_blocks = (ntiles + kGatherTiles - 1) / kGatherTiles;
-    hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks), dim3(kGatherBlock), 0, h->stream, data,
+    hipLaunchKernelGGL((gather_kernel<T, MODE, VEC, ITEMS>), dim3(gather_blocks + (zero_words ? 1u : 0u)),
+                       dim3(kGatherBlock), 0, h->stream, data,
                        update, (long long)n, thr_ptr, thr_val, sc.counts, sc.block_sums,
                        sc.offsets, sc.staging, ntiles, msg_words, cap_pairs, size_prefix, dense_hint ? 0 : 1,
-                       status, slot_pairs);
+                       status, slot_pairs, zero_words, zero_count);
     if (dense_hint) {
         const unsigned redo_blocks = stage_blocks < 2048u ? stage_blocks : 2048u;
         hipLaunchKernelGGL((redo_kernel<T, MODE, VEC, ITEMS>), dim3(redo_blocks), dim3(kBlock), 0, h->stream, data,
@@ -651,6 +718,10 @@ int launch_compact(cx_handle h, void* out_msg, long long out_capacity, const T* 
     const long long cap_pairs = (out_capacity - 8) / kPairBytes;
     const T thr_val = thr_host ? *thr_host : (T)0;
     const T* thr_ptr = thr_host ? nullptr : (d_thr ? d_thr : static_cast<const T*>(h->d_thr));
+    if (h->pending_pick.active && (mode != 0 || no_alloc || thr_ptr != h->pending_pick.thr_out)) {
+        int rc = launch_pending_pick<T>(h);  // not a pass that can make the pick itself
+        if (rc != CX_OK) return rc;
+    }
 
     constexpr int kVec = 16 / (int)sizeof(T);
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(update)) & 15u) == 0;
