@@ -73,7 +73,39 @@ __global__ __launch_bounds__(kBlock) void select_final_kernel(SelectState* st, u
 
 // One histogram pass over the keys described by (vec, add, idx).  SMODE: 0 whole vector,
 // 1 strided, 2 indexed.  The first `nblocks` blocks of the grid share the keys; the others leave.
-template <typename T, int SMODE, bool HAS_ADD, int VEC>
+// Keys into the block's histogram.  Zero keys are counted in a register and go in once per wavefront:
+// the zeros of a sparse gradient would otherwise queue up 64 deep on one LDS address (three passes over
+// 2^20 zeros: 37 us against 22 us for normal data; over 10^8: 1.0 ms against 0.48 ms; with this 21 us and
+// 0.23 ms, and vectors of 90 % zeros 20 us and 0.23 ms against 25 us and 0.47 ms).  It costs normal data
+// 1.2 us per selection of 2^20 keys.  Measured alternatives on 2^20 normal keys: a wavefront's equal
+// digits put together with ballots +4 us per selection, a thread's equal digits in a row as one atomic
+// +2.5 us.
+struct DigitCounter {
+    unsigned zeros = 0u;
+    template <typename KEY>
+    __device__ __forceinline__ void count(unsigned* lds_hist, bool counted, KEY key, unsigned digit) {
+        zeros += (counted && key == (KEY)0) ? 1u : 0u;
+        if (counted && key != (KEY)0) atomicAdd(&lds_hist[digit], 1u);
+    }
+    // every lane of the wavefront must call this
+    __device__ __forceinline__ void flush(unsigned* lds_hist) {
+        unsigned z = zeros;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
+        if ((threadIdx.x & 63) == 0 && z) atomicAdd(&lds_hist[0], z);
+        zeros = 0u;
+    }
+};
+
+// Loads in flight per thread and threads per block of select_hist_kernel.  Measured as three chained passes
+// over r + g, normal data, 2^18 / 2^20 / 2^22 / 10^8 keys: one load at a time, 256 threads 19.3 / 26.4 / 40.9 /
+// 464 us; four loads, 256 threads 19.7 / 23.9 / 36.0 / 489; four loads, 512 threads 19.0 / 22.3 / 32.8 / 469;
+// four loads, 1024 threads 18.1 / 21.6 / 30.4 / 439 (a pass with about 128 blocks leaves a SIMD one wavefront of
+// 256-thread blocks, and its arithmetic between the LDS atomics is then exposed); eight loads: no better.
+constexpr int kHistUnroll = 4;
+constexpr int kHistBlock = 1024;
+
+template <typename T, int SMODE, bool HAS_ADD, int VEC, int BLOCK>
 __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __restrict__ add,
                                           const int* __restrict__ idx, long long m, int n, float stepsize,
                                           SelectState* __restrict__ st, int p, unsigned long long rank0,
@@ -81,7 +113,7 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
     using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
-    __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    __shared__ unsigned long long s_above, s_sum[BLOCK / 64];
     if (blockIdx.x >= nblocks) return;
     // chained passes: every block redoes the cheap pick over the previous pass's complete histogram
     // (issuing the first round of loads before the pick was measured: 0.1 to 0.2 us per step on 61 706 and
@@ -91,10 +123,10 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
     s.mask = 0ull;
     s.rank = rank0;
     if (p > 0) {
-        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above, prev_hist);
+        s = state_entering_pass<T, BLOCK>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above, prev_hist);
         if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
     }
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) lds_hist[b] = 0u;
     __syncthreads();
 
     const key_t prefix = (key_t)s.prefix;
@@ -102,11 +134,31 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
     int shift, bits;
     pass_digits_dev<T>(p, shift, bits);
     const unsigned digit_mask = (1u << bits) - 1u;
-    const long long stride = (long long)nblocks * kBlock;
+    const long long stride = (long long)nblocks * BLOCK;
+    DigitCounter run;
 
     if (SMODE == 0 && VEC > 1) {
         const long long nvec = m / VEC;
-        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < nvec; i += stride) {
+        long long i = (long long)blockIdx.x * BLOCK + threadIdx.x;
+        // kHistUnroll rounds of loads in flight per thread
+        for (; i + (kHistUnroll - 1) * stride < nvec; i += kHistUnroll * stride) {
+            Pack<T, VEC> x[kHistUnroll], y[kHistUnroll];
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u) {
+                x[u] = reinterpret_cast<const Pack<T, VEC>*>(vec)[i + u * stride];
+                if (HAS_ADD) y[u] = reinterpret_cast<const Pack<T, VEC>*>(add)[i + u * stride];
+            }
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u) {
+#pragma unroll
+                for (int c = 0; c < VEC; ++c) {
+                    const T v = HAS_ADD ? (T)(x[u].x[c] + y[u].x[c]) : x[u].x[c];
+                    const key_t k = key_of(v);
+                    run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
+                }
+            }
+        }
+        for (; i < nvec; i += stride) {
             Pack<T, VEC> x = reinterpret_cast<const Pack<T, VEC>*>(vec)[i];
             if (HAS_ADD) {
                 Pack<T, VEC> y = reinterpret_cast<const Pack<T, VEC>*>(add)[i];
@@ -116,18 +168,18 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
 #pragma unroll
             for (int c = 0; c < VEC; ++c) {
                 const key_t k = key_of(x.x[c]);
-                if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+                run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
             }
         }
         // tail elements
-        for (long long i = nvec * VEC + (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
+        for (long long i = nvec * VEC + (long long)blockIdx.x * BLOCK + threadIdx.x; i < m; i += stride) {
             T v = vec[i];
             if (HAS_ADD) v = (T)(v + add[i]);
             const key_t k = key_of(v);
-            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+            run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
         }
     } else {
-        for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < m; i += stride) {
+        for (long long i = (long long)blockIdx.x * BLOCK + threadIdx.x; i < m; i += stride) {
             long long p;
             bool ok = true;
             if (SMODE == 0) {
@@ -145,22 +197,23 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
             T v = vec[p];
             if (HAS_ADD) v = (T)(v + add[p]);
             const key_t k = ok ? key_of(v) : (key_t)0;
-            if ((k & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k >> shift) & digit_mask], 1u);
+            run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
         }
     }
+    run.flush(lds_hist);
     __syncthreads();
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) {
         const unsigned c = lds_hist[b];
         if (c) atomicAdd(&st->pass_hist[p][b], c);
     }
 }
 
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
-__global__ __launch_bounds__(kBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
-                                                             const int* __restrict__ idx, long long m, int n,
-                                                             float stepsize, SelectState* __restrict__ st, int p,
-                                                             unsigned long long rank0) {
-    hist_pass<T, SMODE, HAS_ADD, VEC>(vec, add, idx, m, n, stepsize, st, p, rank0, gridDim.x);
+__global__ __launch_bounds__(kHistBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+                                                                 const int* __restrict__ idx, long long m, int n,
+                                                                 float stepsize, SelectState* __restrict__ st, int p,
+                                                                 unsigned long long rank0) {
+    hist_pass<T, SMODE, HAS_ADD, VEC, kHistBlock>(vec, add, idx, m, n, stepsize, st, p, rank0, gridDim.x);
 }
 
 // The same pass where the DEVICE decides what is counted: the *cand_count candidate keys (magnitude bit
@@ -183,10 +236,10 @@ __global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __r
         constexpr unsigned kPerBlock = (unsigned)kBlock * VEC * 8u;
         unsigned need = (count + kPerBlock - 1u) / kPerBlock;
         if (need > gridDim.x) need = gridDim.x;
-        hist_pass<T, 0, false, VEC>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
+        hist_pass<T, 0, false, VEC, kBlock>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
                                     st, p, rank0, need, p == 1 ? st->pass_hist[kPasses] : nullptr);
     } else {
-        hist_pass<T, 0, HAS_ADD, VEC>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
+        hist_pass<T, 0, HAS_ADD, VEC, kBlock>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
     }
 }
 
@@ -866,16 +919,17 @@ template <typename T, int SMODE, bool HAS_ADD, int VEC>
 void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long long m, int n, float stepsize, int p,
                  unsigned long long rank0) {
     // Blocks: every block merges its histogram with atomics, few blocks leave memory idle.  Measured,
-    // three passes + pick, with 2 / 4 / 8 / 16 16-byte loads per thread: 150 000 keys 17.0 / 17.9 / 20.6 /
-    // 26.3 us, 2^20 keys 28.7 / 23.9 / 23.6 / 27.9 us, 2^22 keys 73.0 / 49.9 / 38.5 / 37.1 us: about 128
-    // blocks while 2 to 16 loads per thread allow it.
-    const long long fine = (long long)kBlock * VEC * 2, coarse = (long long)kBlock * VEC * 16;
+    // three passes + pick, 256-thread blocks with 2 / 4 / 8 / 16 16-byte loads per thread: 150 000 keys 17.0 /
+    // 17.9 / 20.6 / 26.3 us, 2^20 keys 28.7 / 23.9 / 23.6 / 27.9 us, 2^22 keys 73.0 / 49.9 / 38.5 / 37.1 us: about
+    // 128 blocks while 2048 to 65 536 keys per block allow it (again with four loads in flight, 2^20 keys, at
+    // least 64 / 96 / 128 / 256 / 512 blocks: 23.6 / 22.5 / 21.5 / 23.1 / 28.9 us).
+    const long long fine = 256ll * VEC * 2, coarse = (long long)kHistBlock * VEC * 16;
     const long long at_most = (m + fine - 1) / fine, at_least = (m + coarse - 1) / coarse;
     long long blocks = at_least > 128 ? at_least : 128;
     if (blocks > at_most) blocks = at_most;
     if (blocks < 1) blocks = 1;
     if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL((select_hist_kernel<T, SMODE, HAS_ADD, VEC>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
+    hipLaunchKernelGGL((select_hist_kernel<T, SMODE, HAS_ADD, VEC>), dim3((unsigned)blocks), dim3(kHistBlock), 0, h->stream,
                        vec, add, idx, m, n, stepsize, h->sel, p, rank0);
 }
 
@@ -946,11 +1000,12 @@ int ensure_candidates(cx_handle h, size_t need) {
 }
 
 // From how many elements on the whole-vector threshold takes one candidate pass instead of three
-// histogram passes.  Measured on N(0,1) vectors, top 0.1 % / 1 % / 3 %, candidate pass against three
-// passes: 4 Mi elements 43.0 / 46.8 / 50.6 us against 35.7 / 38.8 / 42.8 us, 5 M 45.6 / 49.4 / 53.9
-// against 45.6 / 49.0 / 53.9, 6 M 48.0 / 50.0 / 53.6 against 53.3 / 57.4 / 63.0, 8 Mi 51.8 / 54.9 / 59.1
-// against 67.3 / 72.7 / 80.9.
-constexpr int kCandidatePassMinN = 5 << 20;
+// histogram passes.  Measured on N(0,1) vectors, top 0.1 % / 1 %, candidate pass against three passes:
+// 5 Mi elements 47.0 / 50.5 us against 37.7 / 39.3 us, 6 M 49.0 / 50.6 against 41.4 / 42.7, 8 Mi 50.0 / 51.3
+// against 48.4 / 50.2, 12 M 56.6 / 58.1 against 58.9 / 61.6, 16 Mi 62.3 / 64.4 against 75.2 / 77.7, 32 Mi 77.3 /
+// 78.9 against 129.6 / 130.4; followed by the compress in the same call: 8 Mi 74.0 / 77.4 against 72.3 / 73.0,
+// 12 M 85.5 / 87.8 against 87.9 / 89.4.
+constexpr int kCandidatePassMinN = 10 << 20;
 // candidates kept for a vector of m elements: a sixteenth of it, at least 4 Mi
 inline size_t candidate_capacity(long long m) {
     return (size_t)m / 16 > ((size_t)1 << 22) ? (size_t)m / 16 : ((size_t)1 << 22);
@@ -1220,7 +1275,9 @@ int launch_topk_threshold(cx_handle h, const T* vec, const T* add_vec, int n, co
 template <typename T> int reserve_select(cx_handle h, int n) {
     int rc = ensure_select_keys(h);
     if (rc != CX_OK) return rc;
-    if (n < kCandidatePassMinN) return CX_OK;  // shorter vectors never take the one-pass selections
+    // shorter vectors never take the one-pass selections (cx_ip_compress_topk's single pass can be asked for from
+    // 2^23 elements on: option fused_topk = 2)
+    if (n < kCandidatePassMinN && n < (1 << 23)) return CX_OK;
     const size_t cap = candidate_capacity(n);
     const size_t as_keys = cap * sizeof(typename Elem<T>::key_t), as_pairs = 8 + cap * Elem<T>::pair_words * 4;
     return ensure_candidates(h, as_keys > as_pairs ? as_keys : as_pairs);

@@ -371,7 +371,7 @@ def test_exact_whole_vector_step_can_be_captured_in_a_hip_graph(oracle):
     replays, give the eager result every time, and the eager result is the checker's."""
     from comprex_amd.device import Handle, message_capacity
     rng = np.random.default_rng(43)
-    n = 9_000_001
+    n = 11_000_001
     g_h = rng.laplace(size=n).astype(np.float32)
     g = torch.from_numpy(g_h).cuda()
     rests = torch.zeros(n, device="cuda")

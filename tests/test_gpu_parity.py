@@ -309,9 +309,9 @@ def test_topk_threshold_matches_oracle(dev, oracle, dtype):
 
 def test_exact_threshold_on_both_sides_of_the_candidate_pass_limit(dev, oracle):
     """Whole-vector thresholds just below and at the length from which one candidate pass replaces the
-    three histogram passes (5 Mi elements): the checker's bits on both sides."""
+    three histogram passes (10 Mi elements): the checker's bits on both sides."""
     rng = np.random.default_rng(29)
-    for n in ((5 << 20) - 1, 5 << 20, (5 << 20) + 3):
+    for n in ((10 << 20) - 1, 10 << 20, (10 << 20) + 3):
         v = rng.laplace(size=n).astype(np.float32)
         a = (0.1 * rng.standard_normal(n)).astype(np.float32)
         gv, ga = _gpu(v), _gpu(a)
@@ -328,7 +328,7 @@ def test_exact_threshold_one_pass_bracket_and_fallbacks(dev, oracle, dtype):
     all-equal magnitudes (candidates overflow), a constant vector with a few outliers, and a
     large topK (bracket not attempted).  Same bits as the checker, with the path on and off."""
     rng = np.random.default_rng(19)
-    n = 9_000_001
+    n = 11_000_001
     ds = 1 << 24  # > n: exact mode
     base = (rng.standard_normal(n) * 3).astype(dtype)
     cases = {
@@ -363,7 +363,7 @@ def test_fused_exact_topk_single_pass_and_changes_of_plan(dev, oracle, dtype):
     threshold, small values exactly at the sampled positions), and parameters for which the
     single pass is not attempted (route 0).  Message, residual and threshold: the checker's bits."""
     rng = np.random.default_rng(23)
-    n = 9_000_001
+    n = 11_000_001
     ds = 1 << 24  # > n: whole-vector mode of the reference
     if dtype == np.int32:
         base = rng.integers(-100000, 100001, n).astype(np.int32)

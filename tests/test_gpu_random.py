@@ -179,8 +179,8 @@ def test_random_write_step_across_the_selection_paths(dev, oracle):
     from comprex_amd.device import message_capacity
     rng = np.random.default_rng(99)
     np2t = {np.float32: torch.float32, np.float64: torch.float64, np.int32: torch.int32}
-    sizes = [1, 63, 4097, 40_960, 40_961, 100_000, 262_144, 262_145, 1 << 20, (1 << 22) + 1, (5 << 20) - 1, 5 << 20,
-             (1 << 23) + 1, (20 << 20) - 4, (20 << 20) + 4]
+    sizes = [1, 63, 4097, 40_960, 40_961, 100_000, 262_144, 262_145, 1 << 20, (1 << 22) + 1, (10 << 20) - 1, 10 << 20,
+             12_000_001, (20 << 20) - 4, (20 << 20) + 4]
     routes = set()
     for case, n in enumerate(sizes + sizes):
         dtype = [np.float32, np.float64, np.int32][case % 3]
