@@ -173,7 +173,8 @@ int launch_candidates(cx_handle h, unsigned* cand_words, long long cap_pairs, co
                       const T* d_bound);
 template <typename T>
 int launch_filter(cx_handle h, const unsigned* cand_words, unsigned cand_cap, unsigned long long rank, T* d_thr,
-                  T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result);
+                  T* update, int n, unsigned* msg_words, long long cap_pairs, int* size_prefix, unsigned* d_result,
+                  unsigned long long expected_candidates);
 template <typename T>
 int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, const T* data, T* update, int n,
                          float topK, T* d_thr_out, int* d_size_prefix);

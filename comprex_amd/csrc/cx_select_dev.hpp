@@ -94,7 +94,7 @@ template <typename T> __device__ __forceinline__ void pass_digits_dev(int p, int
 // replaces pass p-1's histogram when those counts were made elsewhere.
 template <typename T, int BLOCK>
 __device__ __forceinline__ PickState state_entering_pass(const SelectState* __restrict__ st, int p,
-                                                         unsigned long long rank0, unsigned* lds_hist,
+                                                         unsigned long long rank0,
                                                          unsigned long long* s_sum, unsigned* s_digit,
                                                          unsigned long long* s_above,
                                                          const unsigned* __restrict__ prev_hist = nullptr) {
@@ -106,12 +106,11 @@ __device__ __forceinline__ PickState state_entering_pass(const SelectState* __re
     } else {
         s = st->pass_state[p - 1];
     }
+    // every thread reads its own bins straight from the global histogram (through LDS first: 0.3 us more per pick)
     const unsigned* counts = prev_hist ? prev_hist : st->pass_hist[p - 1];
-    for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) lds_hist[b] = counts[b];
-    __syncthreads();
     unsigned digit;
     unsigned long long above;
-    block_pick<BLOCK>(lds_hist, s.rank, s_sum, s_digit, s_above, digit, above);
+    block_pick<BLOCK>(counts, s.rank, s_sum, s_digit, s_above, digit, above);
     int shift, bits;
     pass_digits_dev<T>(p - 1, shift, bits);
     s.prefix |= (unsigned long long)digit << shift;

@@ -59,10 +59,9 @@ __global__ __launch_bounds__(kBlock) void select_final_kernel(SelectState* st, u
                                                               T* __restrict__ thr_out) {
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     using key_t = typename Elem<T>::key_t;
-    __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
     __shared__ unsigned long long s_above, s_sum[kBlock / 64];
-    const PickState done = state_entering_pass<T, kBlock>(st, kPasses, rank0, lds_hist, s_sum, &s_digit, &s_above);
+    const PickState done = state_entering_pass<T, kBlock>(st, kPasses, rank0, s_sum, &s_digit, &s_above);
     if (threadIdx.x == 0) {
         T v = value_of((key_t)done.prefix, T());
         if (plus_one) v = (T)(v + 1);
@@ -123,7 +122,7 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
     s.mask = 0ull;
     s.rank = rank0;
     if (p > 0) {
-        s = state_entering_pass<T, BLOCK>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above, prev_hist);
+        s = state_entering_pass<T, BLOCK>(st, p, rank0, s_sum, &s_digit, &s_above, prev_hist);
         if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
     }
     for (int b = threadIdx.x; b < kRadixBins; b += BLOCK) lds_hist[b] = 0u;
@@ -222,8 +221,14 @@ __global__ __launch_bounds__(kHistBlock) void select_hist_kernel(const T* __rest
 // host launches the passes without knowing which way they go.  The grid is sized for the whole
 // vector; over the candidates only the blocks they need stay, and pass 0 has nothing to do: the
 // kernel that collected them left their top-digit counts behind the last pass's histogram.
+// Threads of a block of select_hist_either_kernel and 16-byte loads per thread over the candidates.  Measured as
+// the whole threshold call on 12 M / 32 Mi / 10^8 elements at 1 %: 256 x 8 loads 56 / 79 / 156 us, 256 x 4: 54 / 79 /
+// 159, 512 x 4: 54 / 78 / 156, 1024 x 2: 54 / 79 / 157, 1024 x 8: 58 / 82 / 157 (nothing to choose between them).
+constexpr int kEitherBlock = 256;
+constexpr unsigned kEitherLoads = 8u;
+
 template <typename T, bool HAS_ADD, int VEC>
-__global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __restrict__ vec, const T* __restrict__ add,
+__global__ __launch_bounds__(kEitherBlock) void select_hist_either_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                                     long long m,
                                                                     const typename Elem<T>::key_t* __restrict__ cand,
                                                                     unsigned cap, const unsigned* __restrict__ cand_count,
@@ -233,13 +238,13 @@ __global__ __launch_bounds__(kBlock) void select_hist_either_kernel(const T* __r
     const unsigned count = *cand_count;
     if ((unsigned long long)count > rank0 && count <= cap) {
         if (p == 0) return;
-        constexpr unsigned kPerBlock = (unsigned)kBlock * VEC * 8u;
+        constexpr unsigned kPerBlock = (unsigned)kEitherBlock * VEC * kEitherLoads;
         unsigned need = (count + kPerBlock - 1u) / kPerBlock;
         if (need > gridDim.x) need = gridDim.x;
-        hist_pass<T, 0, false, VEC, kBlock>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
+        hist_pass<T, 0, false, VEC, kEitherBlock>(reinterpret_cast<const T*>(cand), nullptr, nullptr, (long long)count, (int)count, 1.0f,
                                     st, p, rank0, need, p == 1 ? st->pass_hist[kPasses] : nullptr);
     } else {
-        hist_pass<T, 0, HAS_ADD, VEC, kBlock>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
+        hist_pass<T, 0, HAS_ADD, VEC, kEitherBlock>(vec, add, nullptr, m, (int)m, 1.0f, st, p, rank0, gridDim.x);
     }
 }
 
@@ -252,24 +257,31 @@ template <> __device__ __forceinline__ uint64_t pair_key<double>(const unsigned*
     return ((uint64_t)w[1] | ((uint64_t)w[2] << 32)) & 0x7fffffffffffffffull;
 }
 
+// Threads and blocks of select_hist_pairs_kernel: every block merges its histogram with global atomics, so few
+// large blocks.  Measured as the whole single-pass call on 25.6 M elements at 0.1 % / 1 % and on 10^8 at 1 %:
+// 256 x 256 threads 113.4 / 121.9 / 276.4 us, 64 x 1024 110.1 / 117.5 / 270.6, 128 x 1024 109.3 / 115.5 / 265.3,
+// 128 x 512 109.2 / 117.7 / 271.9, 32 x 1024 110.1 / 121.2 / 287.0.
+constexpr int kPairsBlock = 1024;
+constexpr int kPairsBlocks = 128;
+
 template <typename T>
-__global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigned* __restrict__ msg_words, unsigned cap,
+__global__ __launch_bounds__(kPairsBlock) void select_hist_pairs_kernel(const unsigned* __restrict__ msg_words, unsigned cap,
                                                                    SelectState* __restrict__ st, int p,
                                                                    unsigned long long rank0) {
     using key_t = typename Elem<T>::key_t;
     constexpr int PW = Elem<T>::pair_words;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
-    __shared__ unsigned long long s_above, s_sum[kBlock / 64];
+    __shared__ unsigned long long s_above, s_sum[kPairsBlock / 64];
     PickState s;
     s.prefix = 0ull;
     s.mask = 0ull;
     s.rank = rank0;
     if (p > 0) {
-        s = state_entering_pass<T, kBlock>(st, p, rank0, lds_hist, s_sum, &s_digit, &s_above);
+        s = state_entering_pass<T, kPairsBlock>(st, p, rank0, s_sum, &s_digit, &s_above);
         if (blockIdx.x == 0 && threadIdx.x == 0) st->pass_state[p] = s;
     }
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) lds_hist[b] = 0u;
+    for (int b = threadIdx.x; b < kRadixBins; b += kPairsBlock) lds_hist[b] = 0u;
     __syncthreads();
     const key_t prefix = (key_t)s.prefix;
     const key_t mask = (key_t)s.mask;
@@ -278,10 +290,10 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
     const unsigned digit_mask = (1u << bits) - 1u;
     unsigned m = msg_words[1];
     if (m > cap) m = cap;
-    const unsigned stride = gridDim.x * kBlock;
+    const unsigned stride = gridDim.x * kPairsBlock;
     // whole wavefronts stay in the loop together (hist_add is a cross-lane operation); four
     // independent loads per lane are in flight before the first count
-    for (unsigned i0 = blockIdx.x * kBlock; i0 < m; i0 += 4u * stride) {
+    for (unsigned i0 = blockIdx.x * kPairsBlock; i0 < m; i0 += 4u * stride) {
         key_t k[4];
         bool in[4];
 #pragma unroll
@@ -295,7 +307,7 @@ __global__ __launch_bounds__(kBlock) void select_hist_pairs_kernel(const unsigne
             hist_add(lds_hist, in[q] && (k[q] & mask) == prefix, (unsigned)(k[q] >> shift) & digit_mask);
     }
     __syncthreads();
-    for (int b = threadIdx.x; b < kRadixBins; b += kBlock) {
+    for (int b = threadIdx.x; b < kRadixBins; b += kPairsBlock) {
         const unsigned c = lds_hist[b];
         if (c) atomicAdd(&st->pass_hist[p][b], c);
     }
@@ -1153,10 +1165,10 @@ int select_rank_bracketed(cx_handle h, const T* vec, const T* add_vec, int m, un
     if (blocks > 2048) blocks = 2048;
     for (int q = 0; q < kPasses; ++q) {
         if (add_vec)
-            hipLaunchKernelGGL((select_hist_either_kernel<T, true, kVec>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
+            hipLaunchKernelGGL((select_hist_either_kernel<T, true, kVec>), dim3((unsigned)blocks), dim3(kEitherBlock), 0, h->stream,
                                vec, add_vec, (long long)m, cand, (unsigned)cap, d_count, h->sel, q, rank);
         else
-            hipLaunchKernelGGL((select_hist_either_kernel<T, false, kVec>), dim3((unsigned)blocks), dim3(kBlock), 0, h->stream,
+            hipLaunchKernelGGL((select_hist_either_kernel<T, false, kVec>), dim3((unsigned)blocks), dim3(kEitherBlock), 0, h->stream,
                                vec, add_vec, (long long)m, cand, (unsigned)cap, d_count, h->sel, q, rank);
     }
     *done = 1;
@@ -1226,17 +1238,17 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
     if (rc != CX_OK) return rc;
     // 3. threshold among the candidates
     // (chained passes: the pick after each pass is redone by every block of the next kernel, the
-    // last one by the filter, which also writes the threshold and clears the histograms).  Blocks per
-    // pass, measured as the whole call on 100 M fp32 elements at 1 % / on 25.6 M at 0.1 %: 64 blocks
-    // 0.340 ms / 120 us, 128 0.304 / 117, 256 0.297 / 121, 512 0.304 / 123, 1024 0.318 / 124.
+    // last one by the filter, which also writes the threshold and clears the histograms; block shape:
+    // see kPairsBlock).
     constexpr int kPasses = (Elem<T>::key_bits + kRadixBits - 1) / kRadixBits;
     for (int p = 0; p < kPasses; ++p)
-        hipLaunchKernelGGL(select_hist_pairs_kernel<T>, dim3(256), dim3(kBlock), 0, h->stream, cand_words, (unsigned)cap,
+        hipLaunchKernelGGL(select_hist_pairs_kernel<T>, dim3(kPairsBlocks), dim3(kPairsBlock), 0, h->stream, cand_words, (unsigned)cap,
                            h->sel, p, rank);
     CX_HIP(hipGetLastError());
     // 4. message + residual
     rc = launch_filter<T>(h, cand_words, (unsigned)cap, rank, d_thr_out, update, n, static_cast<unsigned*>(out_msg),
-                          (out_capacity - 8) / (4 * PW), d_size_prefix, d_result);
+                          (out_capacity - 8) / (4 * PW), d_size_prefix, d_result,
+                          (unsigned long long)((double)sample_rank / (double)kSample * (double)n));
     if (rc != CX_OK) return rc;
     CX_HIP(hipMemcpyAsync(h->h_pinned + 12, d_result, 2 * sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
     CX_HIP(hipStreamSynchronize(h->stream));
