@@ -606,9 +606,16 @@ __global__ __launch_bounds__(kFinishBlock) void select_finish_kernel(const typen
                     if ((k1 & mask) == prefix) atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 }
             } else {
+                // zero keys are counted in a register and go in once per wavefront: a vector of (mostly) zeros
+                // would otherwise queue every key up on one LDS address (61 706 zeros: 134 us)
+                unsigned zeros = 0u;
                 scan_matching<key_t>(src, src_n, prefix, mask, [&](key_t k1) {
-                    atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
+                    if (k1 == (key_t)0) ++zeros;
+                    else atomicAdd(&lds_hist[(unsigned)(k1 >> shift) & digit_mask], 1u);
                 });
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) zeros += __shfl_xor(zeros, off, 64);
+                if (lane == 0 && zeros) atomicAdd(&lds_hist[0], zeros);
             }
             __syncthreads();
         }
