@@ -1221,10 +1221,10 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
     const bool vec_ok = ((reinterpret_cast<uintptr_t>(data) | reinterpret_cast<uintptr_t>(update)) & 15u) == 0;
     const bool msg_ok = out_msg && (reinterpret_cast<uintptr_t>(out_msg) & 3u) == 0 && out_capacity >= 8;
     // From how many elements on?  Measured on N(0,1) vectors, top 0.1 % / 1 %, this single pass (which
-    // ends with a wait) against the one-pass threshold followed by the compress (which never wait):
-    // 8 Mi elements 85 / 90 us against 73 / 77 us, 12 M 89 / 97 against 85 / 88, 16 Mi 99 / 106 against
-    // 98 / 101, 25.6 M 118 / 125 against 124 / 127, 32 Mi 132 / 138 against 145 / 148, 64 Mi 192 / 211
-    // against 245 / 250.  (Option fused_topk = 2 takes the single pass from 2^23 elements on.)
+    // ends with a wait) against the threshold followed by the compress (which never wait):
+    // 8 Mi elements 73 / 81 us against 69 / 70 us, 12 M 81 / 87 against 81 / 84, 16 Mi 89 / 97 against
+    // 94 / 96, 20 Mi 100 / 108 against 109 / 111, 25.6 M 107 / 114 against 121 / 123, 32 Mi 119 / 129 against
+    // 142 / 146.  (Option fused_topk = 2 takes the single pass from 2^23 elements on.)
     constexpr int kSinglePassMinN = 20 << 20;
     const int single_pass_from = h->fused_topk >= 2 ? (1 << 23) : kSinglePassMinN;
     const bool single_pass = h->fused_topk && data && update && n >= single_pass_from && pos > 0 && vec_ok && msg_ok &&
