@@ -108,7 +108,8 @@ template <typename T, int SMODE, bool HAS_ADD, int VEC, int BLOCK>
 __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __restrict__ add,
                                           const int* __restrict__ idx, long long m, int n, float stepsize,
                                           SelectState* __restrict__ st, int p, unsigned long long rank0,
-                                          unsigned nblocks, const unsigned* __restrict__ prev_hist = nullptr) {
+                                          unsigned nblocks, const unsigned* __restrict__ prev_hist = nullptr,
+                                          typename Elem<T>::key_t* __restrict__ keys_out = nullptr) {
     using key_t = typename Elem<T>::key_t;
     __shared__ unsigned lds_hist[kRadixBins];
     __shared__ unsigned s_digit;
@@ -178,9 +179,10 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
             run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
         }
     } else {
-        for (long long i = (long long)blockIdx.x * BLOCK + threadIdx.x; i < m; i += stride) {
+        // where key i is read from
+        auto position = [&](long long i, bool& ok) -> long long {
             long long p;
-            bool ok = true;
+            ok = true;
             if (SMODE == 0) {
                 p = i;
             } else if (SMODE == 1) {
@@ -193,9 +195,35 @@ __device__ __forceinline__ void hist_pass(const T* __restrict__ vec, const T* __
                 ok = p >= 0 && p < (long long)n;  // positions outside the vector count as magnitude 0
                 if (!ok) p = 0;
             }
+            return p;
+        };
+        long long i = (long long)blockIdx.x * BLOCK + threadIdx.x;
+        // kHistUnroll keys' dependent loads (position, then the values there) in flight per thread
+        for (; i + (kHistUnroll - 1) * stride < m; i += kHistUnroll * stride) {
+            long long p[kHistUnroll];
+            bool ok[kHistUnroll];
+            T v[kHistUnroll];
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u) p[u] = position(i + u * stride, ok[u]);
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u) {
+                v[u] = vec[p[u]];
+                if (HAS_ADD) v[u] = (T)(v[u] + add[p[u]]);
+            }
+#pragma unroll
+            for (int u = 0; u < kHistUnroll; ++u) {
+                const key_t k = ok[u] ? key_of(v[u]) : (key_t)0;
+                if (keys_out) keys_out[i + u * stride] = k;
+                run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
+            }
+        }
+        for (; i < m; i += stride) {
+            bool ok;
+            const long long p = position(i, ok);
             T v = vec[p];
             if (HAS_ADD) v = (T)(v + add[p]);
             const key_t k = ok ? key_of(v) : (key_t)0;
+            if (keys_out) keys_out[i] = k;
             run.count(lds_hist, (k & mask) == prefix, k, (unsigned)(k >> shift) & digit_mask);
         }
     }
@@ -211,8 +239,9 @@ template <typename T, int SMODE, bool HAS_ADD, int VEC>
 __global__ __launch_bounds__(kHistBlock) void select_hist_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                                  const int* __restrict__ idx, long long m, int n,
                                                                  float stepsize, SelectState* __restrict__ st, int p,
-                                                                 unsigned long long rank0) {
-    hist_pass<T, SMODE, HAS_ADD, VEC, kHistBlock>(vec, add, idx, m, n, stepsize, st, p, rank0, gridDim.x);
+                                                                 unsigned long long rank0,
+                                                                 typename Elem<T>::key_t* __restrict__ keys_out) {
+    hist_pass<T, SMODE, HAS_ADD, VEC, kHistBlock>(vec, add, idx, m, n, stepsize, st, p, rank0, gridDim.x, nullptr, keys_out);
 }
 
 // The same pass where the DEVICE decides what is counted: the *cand_count candidate keys (magnitude bit
@@ -945,7 +974,7 @@ template <typename T> __global__ void set_scalar_kernel(T* out, T v) { *out = v;
 
 template <typename T, int SMODE, bool HAS_ADD, int VEC>
 void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long long m, int n, float stepsize, int p,
-                 unsigned long long rank0) {
+                 unsigned long long rank0, typename Elem<T>::key_t* keys_out) {
     // Blocks: every block merges its histogram with atomics, few blocks leave memory idle.  Measured,
     // three passes + pick, 256-thread blocks with 2 / 4 / 8 / 16 16-byte loads per thread: 150 000 keys 17.0 /
     // 17.9 / 20.6 / 26.3 us, 2^20 keys 28.7 / 23.9 / 23.6 / 27.9 us, 2^22 keys 73.0 / 49.9 / 38.5 / 37.1 us: about
@@ -958,20 +987,20 @@ void launch_hist(cx_handle h, const T* vec, const T* add, const int* idx, long l
     if (blocks < 1) blocks = 1;
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL((select_hist_kernel<T, SMODE, HAS_ADD, VEC>), dim3((unsigned)blocks), dim3(kHistBlock), 0, h->stream,
-                       vec, add, idx, m, n, stepsize, h->sel, p, rank0);
+                       vec, add, idx, m, n, stepsize, h->sel, p, rank0, keys_out);
 }
 
 template <typename T, bool HAS_ADD>
 void dispatch_hist(cx_handle h, int smode, bool vec_ok, const T* vec, const T* add, const int* idx, long long m, int n,
-                   float stepsize, int p, unsigned long long rank0) {
+                   float stepsize, int p, unsigned long long rank0, typename Elem<T>::key_t* keys_out = nullptr) {
     constexpr int kVec = 16 / (int)sizeof(T);
     if (smode == kSampleFull) {
-        if (vec_ok) launch_hist<T, 0, HAS_ADD, kVec>(h, vec, add, idx, m, n, stepsize, p, rank0);
-        else launch_hist<T, 0, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
+        if (vec_ok) launch_hist<T, 0, HAS_ADD, kVec>(h, vec, add, idx, m, n, stepsize, p, rank0, nullptr);
+        else launch_hist<T, 0, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0, nullptr);
     } else if (smode == kSampleStrided) {
-        launch_hist<T, 1, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
+        launch_hist<T, 1, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0, keys_out);
     } else {
-        launch_hist<T, 2, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0);
+        launch_hist<T, 2, HAS_ADD, 1>(h, vec, add, idx, m, n, stepsize, p, rank0, keys_out);
     }
 }
 
@@ -1118,11 +1147,24 @@ int select_rank(cx_handle h, const T* vec, const T* add_vec, int n, const int* d
     const bool vec_ok =
         ((reinterpret_cast<uintptr_t>(vec) | reinterpret_cast<uintptr_t>(add_vec)) & 15u) == 0;  // null add is aligned
     // chained radix passes (no pick launch in between), then the last pick
+    // A large sample (more keys than the two launches take) is gathered once: pass 0 leaves the keys in the
+    // candidate buffer and the later passes read them from there, consecutive, instead of following the
+    // positions again (10^6 positions in 10^8 elements: 37 us per gathering pass, random reads of two vectors).
+    // Only where the buffer cx_reserve sizes for a vector of n elements holds them.
+    key_t* cached = nullptr;
+    if (sample_mode != kSampleFull && n >= (1 << 23) && (size_t)m <= candidate_capacity(n)) {
+        int rc_cand = ensure_candidates(h, candidate_capacity(n) * sizeof(key_t));
+        if (rc_cand != CX_OK) return rc_cand;
+        cached = static_cast<key_t*>(h->cand);
+    }
     for (int p = 0; p < kPasses; ++p) {
-        if (add_vec)
-            dispatch_hist<T, true>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank);
+        if (cached && p > 0)
+            dispatch_hist<T, false>(h, kSampleFull, true, reinterpret_cast<const T*>(cached), nullptr, nullptr, (long long)m,
+                                    m, 1.0f, p, rank);
+        else if (add_vec)
+            dispatch_hist<T, true>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank, cached);
         else
-            dispatch_hist<T, false>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank);
+            dispatch_hist<T, false>(h, sample_mode, vec_ok, vec, add_vec, d_idx, (long long)m, n, stepsize, p, rank, cached);
     }
     return finish_chained<T>(h, rank, plus_one, d_thr_out);
 }

@@ -473,6 +473,37 @@ def test_topk_threshold_indexed_and_device_slot(dev, oracle):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_sampled_threshold_with_more_samples_than_the_two_launches_take(dev, oracle, dtype):
+    """More than 2^18 sample positions, host-supplied or strided: radix passes over the sample.  On a
+    vector long enough for the handle's candidate buffer the first pass leaves the gathered keys there
+    and the later passes read them back; on a shorter one every pass follows the positions.  Ties,
+    positions outside the vector (magnitude 0) and both orders of the positions: the checker's bits."""
+    rng = np.random.default_rng(61)
+    for n in (9_000_001, 3_000_000):
+        v = _rand(rng, n, dtype)
+        v[rng.integers(0, n, n // 50)] *= 40
+        a = _rand(rng, n, dtype, 0.25)
+        if dtype != np.int32:
+            v = (np.round(v * 8) / 8).astype(dtype)  # ties
+        v[0] = a[0] = 0  # where the checker looks for a position outside the vector (the reference would read out of bounds)
+        gv, ga = _gpu(v), _gpu(a)
+        for m, topk in ((300_000, 0.02), (600_001, 0.001), (262_145, 0.3)):
+            idx = rng.integers(0, n, m).astype(np.int32)
+            idx[::1000] = n + 5
+            idx[1::1000] = -1
+            for order in ("given", "sorted"):
+                if order == "sorted":
+                    idx = np.sort(idx)
+                say("large sample", dtype.__name__, n, m, topk, order)
+                inside = np.where((idx < 0) | (idx >= n), 0, idx).astype(np.int32)
+                want = oracle.topk_prepare_indexed(v, a, inside, np.float32(topk))
+                assert dev.topk_threshold_indexed(gv, ga, _gpu(idx), np.float32(topk)) == want
+            # strided: ThresholdTopK(topK, m, 1.0) takes m sub-samples
+            assert dev.topk_threshold(gv, ga, np.float32(topk), m, 1.0) == oracle.topk_prepare_with(v, a, np.float32(topk), m, 1.0)
+            assert dev.topk_threshold(gv, None, np.float32(topk), m, 1.0) == oracle.topk_prepare(v, np.float32(topk), m, 1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_sampled_threshold_short_list_and_inputs_that_defeat_it(dev, oracle, dtype):
     """The two-launch select hands its second launch a short list of each block's top keys and
     falls back on the full key array when the list cannot hold the answer: large values
