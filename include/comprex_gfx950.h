@@ -155,8 +155,9 @@ int cx_topk_threshold(cx_handle h, cx_dtype dt, const void* vec, const void* add
                       float topK, int default_subsamples, float subsample_factor,
                       void* d_thr_out, void* h_thr_out);
 /* Same order statistic over m host-chosen sample positions d_idx[0..m) (device int32):
- * keys are vec[idx] (+ add_vec[idx]).  No counterpart in the reference, whose sampling
- * is always strided (src/threshold.hxx:224-240); calc_threshold (:189-205) is unchanged. */
+ * keys are vec[idx] (+ add_vec[idx]); a position outside [0, n) counts as a key of magnitude 0
+ * and is never dereferenced.  No counterpart in the reference, whose sampling is always strided
+ * (src/threshold.hxx:224-240); calc_threshold (:189-205) is unchanged. */
 int cx_topk_threshold_indexed(cx_handle h, cx_dtype dt, const void* vec, const void* add_vec,
                               int n, const int* d_idx, int m, float topK, void* d_thr_out, void* h_thr_out);
 /* Device address of the handle's threshold slot (8 bytes, holds a T). */
