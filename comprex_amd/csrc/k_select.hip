@@ -769,7 +769,6 @@ __global__ __launch_bounds__(kFinishBlock) void select_one_block_kernel(const T*
         atomicOr(&s_or, all_or);
     }
     __syncthreads();
-    const unsigned list_n = (unsigned)m;
     const key_t differ = s_and ^ s_or;
     int lo = differ ? 64 - __clzll((unsigned long long)differ) : 0;  // the bits below this one are still open
     const key_t open_bits = lo >= 8 * (int)sizeof(key_t) ? (key_t)~(key_t)0 : (key_t)(((key_t)1 << lo) - 1);
@@ -819,7 +818,6 @@ __global__ __launch_bounds__(kFinishBlock) void select_one_block_kernel(const T*
             lo = 0;
         }
     }
-    (void)list_n;
     if (t == 0) {
         T v = value_of(prefix, T());
         if (plus_one) v = (T)(v + 1);
