@@ -237,6 +237,54 @@ def config_leg(torch, W, cfg, grad_fn, cpu_seconds, with_cpu, cpu_iters_cap):
     return out
 
 
+def api_leg(torch, n, reps=200):
+    """writeRemote / readRemote_add through the reference's own C symbols (Comprex_*; comprex_amd/pygpi.py binds
+    them as the reference's ComprEx.py does) on device vectors, with the reference's default threshold: a
+    ThresholdTopK of 1 % over 1000 strided samples.  Host time per call, the device kept busy back to back."""
+    from comprex_amd import pygpi as P
+    env = P.GaspiEnvironment(1 << 20)
+    thr, comp = P.ThresholdTopK(0.01), P.CompressorIndexPairs()
+    cs = []
+    for rank in range(2):
+        env.set_rank(rank, 2)
+        c = P.Comprex(env, n, 0.2)
+        c.setThreshold(thr)
+        c.setCompressor(comp)
+        c.connectTo((rank + 1) % 2, (rank + 1) % 2, 5)
+        cs.append(c)
+    g = torch.randn(n, device="cuda")
+    out = torch.zeros(n, device="cuda")
+    env.set_user_stream(torch.cuda.current_stream())
+
+    def pair():
+        cs[0].writeRemote(g)
+        cs[1].readRemote_add(out)
+
+    for _ in range(10):
+        pair()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        pair()
+    torch.cuda.synchronize()
+    pair_us = (time.perf_counter() - t0) / reps * 1e6
+    tw = tr = 0.0
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cs[0].writeRemote(g)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        cs[1].readRemote_add(out)
+        torch.cuda.synchronize()
+        tw += t1 - t0
+        tr += time.perf_counter() - t1
+    del cs, env
+    return {"n": n, "threshold": "ThresholdTopK(0.01): 1000 strided samples", "pair_us": pair_us,
+            "writeRemote_alone_us": tw / reps * 1e6, "readRemote_add_alone_us": tr / reps * 1e6,
+            "what": "pair = writeRemote + readRemote_add back to back; alone = one call and a device wait after it"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -490,6 +538,11 @@ def main():
             extra["configs"]["launches_per_step"] = {
                 "C1": 5, "C2": 5, "C3": 9,
                 "source": "rocprofv3 kernel trace of these legs, profiles/configs_C1_C2_C3_kernel_trace.txt, not this run"}
+            # the reference's calls with its default threshold, through its C symbols
+            extra["reference_api_calls"] = [api_leg(torch, W.C2["n"]), api_leg(torch, W.C1["n"])]
+            for leg in extra["reference_api_calls"]:
+                log("Comprex_writeRemote + Comprex_readRemote_add, n=%d, default threshold: %.1f us per pair (alone: %.1f + %.1f us)"
+                    % (leg["n"], leg["pair_us"], leg["writeRemote_alone_us"], leg["readRemote_add_alone_us"]))
 
         # reduce: 8 simulated ranks' 1 %-dense messages into a 64 Mi dense vector (config C5)
         c5n = W.C5["n"] if n == W.C4["n"] else 1 << 22
