@@ -417,8 +417,6 @@ __device__ __forceinline__ void scan_matching(const KEY* src, unsigned count, KE
     }
 }
 
-constexpr bool kDealKeys = true;
-
 template <typename T, int SMODE, bool HAS_ADD>
 __global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __restrict__ vec, const T* __restrict__ add,
                                                               const int* __restrict__ idx, int m, int n, float stepsize,
@@ -446,8 +444,7 @@ __global__ __launch_bounds__(kFirstBlock) void select_first_kernel(const T* __re
     // sized for an even share of the large keys, could not decide (25.6 M elements in layers, 65 536 strided
     // samples: the second launch 12.1 us, with the keys dealt out 5.9 us).  A wavefront's keys, positions
     // and stores stay consecutive.
-    const long long i = kDealKeys ? ((long long)(t >> 6) * gridDim.x + blockIdx.x) * 64 + (t & 63)
-                                  : (long long)blockIdx.x * kFirstBlock + t;
+    const long long i = ((long long)(t >> 6) * gridDim.x + blockIdx.x) * 64 + (t & 63);
     key_t mine = 0;
     const bool have = i < m;
     if (have) {
