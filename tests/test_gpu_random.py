@@ -218,3 +218,33 @@ def test_random_write_step_across_the_selection_paths(dev, oracle):
             assert r.cpu().numpy().tobytes() == r_h.tobytes(), (case, n)
         routes.add(dev.get_option("fused_topk_taken"))
     assert 1 in routes or 2 in routes  # the single pass was among them
+
+
+def test_write_step_on_sub_vectors_that_are_not_16_byte_aligned(dev, oracle):
+    """cx_ip_write_step on vectors that start 1 or 3 elements into an allocation (scalar loads in every
+    kernel of the step, the last pick of a chained selection made by the compress pass): threshold, message
+    and residual are the checker's, and nothing in front of the sub-vector is touched."""
+    from comprex_amd.device import message_capacity
+    rng = np.random.default_rng(3)
+    np2t = {np.float32: torch.float32, np.float64: torch.float64, np.int32: torch.int32}
+    for dtype in (np.float32, np.float64, np.int32):
+        for n in (4097, 100_003, 1_000_001):
+            for off in (1, 3):
+                for ds in (1 << 30, 1000):
+                    topk = np.float32(rng.choice([0.001, 0.02, 0.2]))
+                    scale = 1000 if dtype == np.int32 else 1
+                    g_full = (rng.standard_normal(n + off) * scale).astype(dtype)
+                    r_full = (0.3 * rng.standard_normal(n + off) * scale).astype(dtype)
+                    g_h, r_h = g_full[off:].copy(), r_full[off:].copy()
+                    gg, rr = torch.from_numpy(g_full).cuda(), torch.from_numpy(r_full).cuda()
+                    say("unaligned write_step", dtype.__name__, n, off, ds, float(topk))
+                    buf = torch.zeros(message_capacity(n, np2t[dtype]), dtype=torch.uint8, device="cuda")
+                    thr_out = torch.zeros(1, dtype=np2t[dtype], device="cuda")
+                    nb = dev.write_step(buf, gg[off:], rr[off:], topk, ds, 10.0, d_thr=thr_out)
+                    want_thr = oracle.topk_prepare_with(r_h, g_h, topk, ds, 10.0)
+                    want = oracle.ip_compress(g_h, r_h, dtype(want_thr))
+                    assert thr_out.cpu().numpy()[0] == dtype(want_thr)
+                    assert nb == want.size and buf[:nb].cpu().numpy().tobytes() == want.tobytes()
+                    back = rr.cpu().numpy()
+                    assert back[off:].tobytes() == r_h.tobytes() and back[:off].tobytes() == r_full[:off].tobytes()
+                    assert gg.cpu().numpy().tobytes() == g_full.tobytes()
