@@ -1303,6 +1303,8 @@ int launch_compress_topk(cx_handle h, void* out_msg, long long out_capacity, con
                           (out_capacity - 8) / (4 * PW), d_size_prefix, d_result,
                           (unsigned long long)((double)sample_rank / (double)kSample * (double)n));
     if (rc != CX_OK) return rc;
+    // (letting the last kernel store the result words in pinned host memory itself, without this copy, was
+    // measured: 1 us or less on a call of 105 us)
     CX_HIP(hipMemcpyAsync(h->h_pinned + 12, d_result, 2 * sizeof(unsigned), hipMemcpyDeviceToHost, h->stream));
     CX_HIP(hipStreamSynchronize(h->stream));
     h->fused_topk_taken = 1;
